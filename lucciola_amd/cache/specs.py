@@ -101,6 +101,26 @@ class PagedKV(CacheNeed):
 
 
 @dataclass(frozen=True)
+class PagedLatent(CacheNeed):
+    """One row of ``width`` entries per token, in pages: what a mixer keeps that rebuilds its keys
+    and values from a small latent (the latent itself and, behind it, whatever else all heads
+    share, such as a rotated key part).  ``window`` as for :class:`PagedKV`.
+
+    Memory per site: ``[pages, page, width]``; any page size."""
+
+    width: int
+    window: Optional[int] = None
+
+    paged = True
+
+    def bytes_per_page(self, page_size: int, dtype: torch.dtype) -> int:
+        return page_size * self.width * _element_size(dtype)
+
+    def allocate(self, layout: CacheLayout, dtype: torch.dtype, device):
+        return torch.zeros((layout.kernel_pages, layout.kernel_page, self.width), dtype=dtype, device=device)
+
+
+@dataclass(frozen=True)
 class FixedState(CacheNeed):
     """A tensor of fixed shape per live request: ``[max_seqs, *shape]``, indexed by the
     request's slot and zeroed when a request starts."""

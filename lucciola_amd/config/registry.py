@@ -73,6 +73,7 @@ POSITION_ENCODINGS: Registry[type] = Registry("position encoding")
 BLOCKS: Registry[type] = Registry("block arrangement")
 EMBEDDINGS: Registry[type] = Registry("embedding")
 HEADS: Registry[type] = Registry("output head")
+STREAM_STEPS: Registry[type] = Registry("stream step")
 
 # the families a block's slots may name
 FAMILIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
@@ -81,7 +82,9 @@ FAMILIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
 
 def architecture_for(config_dict: Dict[str, Any]) -> Architecture:
     names = config_dict.get("architectures")
+    if not names and isinstance(config_dict.get("architecture"), str):
+        names = [config_dict["architecture"]]      # some families name their one class in the singular
     if not names or not isinstance(names, (list, tuple)):
-        raise RegistryError("config.json: 'architectures' is missing or empty; known: "
+        raise RegistryError("config.json: 'architectures' (or 'architecture') is missing or empty; known: "
                             + ", ".join(ARCHITECTURES.names()))
     return ARCHITECTURES.get(str(names[0]))

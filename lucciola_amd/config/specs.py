@@ -37,6 +37,11 @@ class LayerSpec:
     names: Dict[str, str]
 
 
+def mixer_only_layer(mixer: PartSpec, mixer_norm: PartSpec, names: Dict[str, str]) -> LayerSpec:
+    """A layer that is a mixer behind its norm and nothing else (``prenorm_mixer``)."""
+    return LayerSpec("prenorm_mixer", {"mixer": mixer, "mixer_norm": mixer_norm}, names)
+
+
 def prenorm_layer(mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
                   feed_forward_norm: PartSpec, names: Dict[str, str]) -> LayerSpec:
     """A layer in the pre-norm residual arrangement (``prenorm_residual``)."""
@@ -55,6 +60,11 @@ class RunEntry:
 
     layer: int
     cache_of: Optional[int] = None
+    # something done to the residual stream right before the layer runs at this site (a vector
+    # that marks the pass of a repeated stack, ...): a part of the ``stream_step`` family, and
+    # the checkpoint names of its tensors
+    before: Optional[PartSpec] = None
+    before_names: Optional[Dict[str, str]] = None
 
 
 @dataclass(frozen=True)

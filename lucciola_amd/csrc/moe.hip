@@ -1,0 +1,159 @@
+// The routing of a mixture of experts, on the device from the router's logits to the weighted
+// sum of the experts' outputs; the host never sees a count.
+//   scores    s = softmax(z) over all experts (float32)
+//   choice    the `top` largest scores (the lower index wins a tie)
+//   weights   the chosen scores, divided by their sum + eps where asked
+//   lists     the (token, choice) pairs sorted by expert: expert e owns the sorted rows
+//             row_start[e] .. row_start[e + 1] - 1, tile_start[e] counts the tiles of `tile` rows of
+//             the experts before it (the grouped product's work list), sorted_token[row] is the
+//             row's token and entry_row[token * top + k] the row of a token's k-th choice
+//   combine   out[t] = sum_k weight[t][k] * y[entry_row[t][k]], k in the order of the choice
+// A sorted row's value does not depend on where in its expert's stretch it lies, so the order in
+// which the pairs of one expert arrive (atomic counters) changes no result.
+#include "common.h"
+
+namespace lc {
+
+constexpr int MOE_MAX_EXPERTS = 512;      // 8 a lane of the routing wave
+constexpr int MOE_PER_LANE = MOE_MAX_EXPERTS / kWave;
+
+// One wave per token.
+__global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restrict__ logits, int E, int top,
+                                                         int renormalise, float eps, int* __restrict__ ids,
+                                                         float* __restrict__ weights) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (size_t)t * E;
+    float s[MOE_PER_LANE];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i) {
+        const int e = lane + kWave * i;
+        s[i] = e < E ? z[e] : -INFINITY;
+        m = fmaxf(m, s[i]);
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i) {
+        s[i] = lane + kWave * i < E ? expf(s[i] - m) : -1.f;     // -1: no expert, below every score
+        sum += fmaxf(s[i], 0.f);
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i)
+        if (s[i] >= 0.f) s[i] = s[i] / sum;
+    float picked_sum = 0.f, mine = 0.f;       // lane k keeps the k-th choice's score
+    for (int k = 0; k < top; ++k) {
+        float best = -1.f;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (s[i] > best) { best = s[i]; at = lane + kWave * i; }     // a lane's experts in rising order
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, kWave);
+            const int oa = __shfl_xor(at, off, kWave);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (lane + kWave * i == at) s[i] = -1.f;
+        if (lane == 0) ids[(size_t)t * top + k] = at;
+        if (lane == k) mine = best;
+        picked_sum += best;
+    }
+    const float div = renormalise ? picked_sum + eps : 1.f;
+    if (lane < top) weights[(size_t)t * top + lane] = mine / div;
+}
+
+// One workgroup: counts, the two running sums, and every pair's sorted row.
+__global__ __launch_bounds__(1024) void moe_lists_kernel(const int* __restrict__ ids, int n, int top, int E,
+                                                         int tile, int* __restrict__ row_start,
+                                                         int* __restrict__ tile_start,
+                                                         int* __restrict__ sorted_token,
+                                                         int* __restrict__ entry_row) {
+    __shared__ int counts[MOE_MAX_EXPERTS];
+    __shared__ int cursor[MOE_MAX_EXPERTS];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) counts[e] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) atomicAdd(&counts[ids[i]], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int rows = 0, tiles = 0;
+        for (int e = 0; e < E; ++e) {
+            row_start[e] = rows;
+            tile_start[e] = tiles;
+            cursor[e] = rows;
+            rows += counts[e];
+            tiles += (counts[e] + tile - 1) / tile;
+        }
+        row_start[E] = rows;
+        tile_start[E] = tiles;
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) {
+        const int row = atomicAdd(&cursor[ids[i]], 1);
+        sorted_token[row] = i / top;
+        entry_row[i] = row;
+    }
+}
+
+template <typename T>
+__global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
+                                   const int* __restrict__ entry_row, int top, int n, T* __restrict__ out) {
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float total = 0.f;
+        for (int k = 0; k < top; ++k)
+            total = fmaf(weights[(size_t)t * top + k], y[(size_t)entry_row[(size_t)t * top + k] * n + i], total);
+        out[(size_t)t * n + i] = from_f32<T>(total);
+    }
+}
+
+}  // namespace lc
+
+using namespace lc;
+
+LC_API int lc_moe_max_experts(void) { return MOE_MAX_EXPERTS; }
+
+// logits float32 [T, E] -> ids int32 [T, top], weights float32 [T, top]
+LC_API int lc_moe_route(const float* logits, int T, int E, int top, int renormalise, float eps, int* ids,
+                        float* weights, hipStream_t stream) {
+    LC_CHECK(T >= 0 && E > 0 && top > 0 && top <= E, "moe route: bad sizes T=%d E=%d top=%d", T, E, top);
+    LC_CHECK(E <= MOE_MAX_EXPERTS, "moe route: %d experts are above the supported %d", E, MOE_MAX_EXPERTS);
+    LC_CHECK(top <= kWave, "moe route: %d choices a token are above the supported %d", top, kWave);
+    if (T == 0) return 0;
+    LC_CHECK(logits && ids && weights, "moe route: null pointer");
+    moe_route_kernel<<<T, kWave, 0, stream>>>(logits, E, top, renormalise, eps, ids, weights);
+    LC_LAUNCH_CHECK("moe_route");
+    return 0;
+}
+
+// ids [T * top] -> row_start, tile_start [E + 1], sorted_token [T * top], entry_row [T * top]
+LC_API int lc_moe_lists(const int* ids, int T, int top, int E, int tile, int* row_start, int* tile_start,
+                        int* sorted_token, int* entry_row, hipStream_t stream) {
+    LC_CHECK(T >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && tile > 0, "moe lists: bad sizes");
+    LC_CHECK(ids && row_start && tile_start && sorted_token && entry_row, "moe lists: null pointer");
+    LC_CHECK((long long)T * top < (1ll << 31), "moe lists: too many rows");
+    moe_lists_kernel<<<1, 1024, 0, stream>>>(ids, T * top, top, E, tile, row_start, tile_start, sorted_token, entry_row);
+    LC_LAUNCH_CHECK("moe_lists");
+    return 0;
+}
+
+// y float32 [T * top, n] -> out [T, n]
+LC_API int lc_moe_combine(const float* y, const float* weights, const int* entry_row, int T, int top, int n,
+                          void* out, int dt, hipStream_t stream) {
+    LC_CHECK(T >= 0 && top > 0 && n > 0, "moe combine: bad sizes");
+    if (T == 0) return 0;
+    LC_CHECK(y && weights && entry_row && out, "moe combine: null pointer");
+    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    if (dt == DT_F32)
+        moe_combine_kernel<float><<<T, threads, 0, stream>>>(y, weights, entry_row, top, n, (float*)out);
+    else if (dt == DT_BF16)
+        moe_combine_kernel<bf16><<<T, threads, 0, stream>>>(y, weights, entry_row, top, n, (bf16*)out);
+    else
+        LC_CHECK(false, "moe combine: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("moe_combine");
+    return 0;
+}

@@ -70,6 +70,16 @@ _SIGNATURES = {
     "lc_sample": "pppppiip",
     "lc_sample_workspace": "i",
     "lc_feed_tokens": "pppiip",
+    "lc_dynamic_tanh": "pppppfpiiiip",
+    "lc_stream_add": "ppipiip",
+    "lc_activation": "piiqp",
+    "lc_gemm_grouped": "piqqpipiqqiiiipppiiipqqp",
+    "lc_latent_prepare": "piqiiiiipfppiipppp",
+    "lc_latent_attention": "piiiiippppiifipp",
+    "lc_moe_max_experts": "",
+    "lc_moe_route": "piiiifppp",
+    "lc_moe_lists": "piiiippppp",
+    "lc_moe_combine": "pppiiipip",
 }
 
 
@@ -863,6 +873,243 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
         raise KernelError("swiglu: the input needs an even number of columns")
     out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
     _call("lc_swiglu", _ptr(gu), _ptr(out), _c_int(_dt(gu)), _c_int(T), _c_int(two_i // 2), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ other norms, other feed-forwards
+ACTIVATIONS = {"gelu_tanh": 1, "relu_squared": 2}
+_EPILOGUE_GATE = 3
+
+
+def dynamic_tanh(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor,
+                 alpha: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``tanh(alpha v) * weight + bias`` of the float32 residual stream ``h`` [T, n] with the pending
+    branch output ``delta`` added first (v = h + delta).  Without ``rows``: ``h += delta`` in place and
+    every row is normed; with ``rows`` (int32 [R]): only those rows, ``h`` stays as it is."""
+    _need(h, "dynamic_tanh h", torch.float32, 2)
+    _need(weight, "dynamic_tanh weight", torch.float32, 1)
+    _need(bias, "dynamic_tanh bias", torch.float32, 1)
+    T, n = h.shape
+    if weight.shape[0] != n or bias.shape[0] != n:
+        raise KernelError(f"dynamic_tanh: weight and bias must have {n} entries")
+    if delta is not None:
+        _need(delta, "dynamic_tanh delta", out_dtype, 2)
+        if tuple(delta.shape) != (T, n):
+            raise KernelError(f"dynamic_tanh: delta {tuple(delta.shape)} does not match h {(T, n)}")
+    if rows is not None:
+        _need(rows, "dynamic_tanh rows", torch.int32, 1)
+    R = T if rows is None else rows.shape[0]
+    out = torch.empty((R, n), dtype=out_dtype, device=h.device)
+    _call("lc_dynamic_tanh", _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(bias), float(alpha), _ptr(out),
+          _dt(out), R, n, 1 if (rows is None and delta is not None) else 0, _stream())
+    return out
+
+
+def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], vector: torch.Tensor) -> None:
+    """``h[t] += delta[t] + vector`` for every row of the float32 residual stream ``h`` [T, n]."""
+    _need(h, "stream_add h", torch.float32, 2)
+    _need(vector, "stream_add vector", torch.float32, 1)
+    T, n = h.shape
+    if vector.shape[0] != n:
+        raise KernelError(f"stream_add: a vector of {vector.shape[0]} entries for rows of {n}")
+    if delta is not None:
+        _need(delta, "stream_add delta", None, 2)
+        if tuple(delta.shape) != (T, n):
+            raise KernelError(f"stream_add: delta {tuple(delta.shape)} does not match h {(T, n)}")
+    _call("lc_stream_add", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(vector), T, n,
+          _stream())
+
+
+def activation(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """``x`` through one of ACTIVATIONS, in place; returns ``x``."""
+    _need(x, "activation x")
+    _call("lc_activation", _ptr(x), _dt(x), ACTIVATIONS[kind], x.numel(), _stream())
+    return x
+
+
+def gemm_act(x, w: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """``act(x . w^T)``: the first product of a two-matrix feed-forward with its activation."""
+    return activation(gemm(x, w, out_dtype), kind)
+
+
+@dataclass
+class Strided:
+    """Equal stretches of the columns of a 2-D tensor, one per group: group g owns the columns
+    ``column + g * group`` onwards (the heads side by side in a row of projections)."""
+
+    tensor: torch.Tensor
+    column: int
+    group: int
+
+    def pointer(self) -> ctypes.c_void_p:
+        return ctypes.c_void_p(self.tensor.data_ptr() + self.column * self.tensor.element_size())
+
+
+def _check_strided(s: Strided, what: str, rows: int, groups: int, width: int, dtype=None) -> None:
+    _need(s.tensor, what, dtype, 2)
+    if s.tensor.shape[0] < rows or s.column < 0 or s.column + (groups - 1) * s.group + width > s.tensor.shape[1]:
+        raise KernelError(f"{what}: {groups} groups of {width} columns from column {s.column}, {s.group} apart, "
+                          f"and {rows} rows do not fit {tuple(s.tensor.shape)}")
+
+
+def grouped_gemm(x: Strided, w: torch.Tensor, out: Strided, rows: int, gate: Optional[Strided] = None,
+                 activation: Optional[str] = None) -> None:
+    """For every group g: ``out_g = x_g . w[g]^T`` over the first ``rows`` rows, with ``w`` [G, N, K], x_g
+    the K columns of group g of ``x`` and out_g the N columns of group g of ``out`` (a product per
+    head over all tokens, in one launch).  With ``gate``: the result times sigmoid of the gate's
+    entry at the same row and column of its group.  True 32-bit arithmetic whatever the types."""
+    _need(w, "grouped_gemm w", None, 3)
+    G, N, K = w.shape
+    _check_strided(x, "grouped_gemm x", rows, G, K)
+    _check_strided(out, "grouped_gemm out", rows, G, N)
+    epilogue = ACTIVATIONS[activation] if activation else 0
+    if gate is not None:
+        if activation:
+            raise KernelError("grouped_gemm: a gate or an activation, not both")
+        _check_strided(gate, "grouped_gemm gate", rows, G, N, x.tensor.dtype)
+        epilogue = _EPILOGUE_GATE
+    if rows == 0:
+        return
+    _call("lc_gemm_grouped", x.pointer(), _dt(x.tensor), x.tensor.shape[1], x.group, _ptr(w), _dt(w),
+          out.pointer(), _dt(out.tensor), out.tensor.shape[1], out.group, rows, N, K, G, None, None, None, 0,
+          1 if rows <= 16 else 0, epilogue, gate.pointer() if gate is not None else None,
+          gate.tensor.shape[1] if gate is not None else 0, gate.group if gate is not None else 0, _stream())
+
+
+# ------------------------------------------------------------------------------ latent attention
+def latent_prepare(proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int, norm_weight: torch.Tensor,
+                   eps: float, positions: torch.Tensor, rope_table: Optional[torch.Tensor], pairing: str,
+                   cache: torch.Tensor, slots: Optional[torch.Tensor], qa: torch.Tensor) -> None:
+    """What latent attention does to a step's projections ``proj`` [T, heads (dim + rot) + rank + rot
+    (+ more)] before it attends: the ``rank`` entries behind the q heads, divided by their root mean
+    square and times ``norm_weight``, and the ``rot`` entries behind them, rotated at the token's
+    position, go to the token's row of ``cache`` [pages, page, rank + rot] (``slots`` [T]: page *
+    page size + offset; negative or None: no write); every head's ``rot`` query entries, rotated,
+    go to ``qa`` [T, heads (rank + rot)] behind the head's ``rank`` entries (which a product fills).
+    ``rope_table`` [positions, rd] holds cosines, then sines; the first rd entries of a part are
+    rotated, as pairs (2i, 2i + 1) (``pairing`` "interleaved") or (i, i + rd/2) ("half")."""
+    _need(proj, "latent_prepare proj", None, 2)
+    T = proj.shape[0]
+    _need(norm_weight, "latent norm weight", torch.float32, 1)
+    if norm_weight.shape[0] != rank:
+        raise KernelError(f"latent_prepare: norm weight has {norm_weight.shape[0]} entries for a latent of {rank}")
+    _need(qa, "latent_prepare qa", proj.dtype, 2)
+    if tuple(qa.shape) != (T, heads * (rank + rot)):
+        raise KernelError(f"latent_prepare: qa {tuple(qa.shape)} is not [{T}, {heads * (rank + rot)}]")
+    if proj.shape[1] < heads * (dim + rot) + rank + rot:
+        raise KernelError(f"latent_prepare: rows of {proj.shape[1]} entries are too short")
+    rd = 0
+    if rope_table is not None and rot:
+        _need(rope_table, "rope table", torch.float32, 2)
+        _need(positions, "positions", torch.int32, 1)
+        rd = rope_table.shape[1]
+        if positions.shape[0] != T or rd > rot or rd % 2:
+            raise KernelError("latent_prepare: positions or rotary table do not fit")
+    else:
+        rope_table = None
+    if slots is not None:
+        _need(cache, "latent cache", proj.dtype, 3)
+        _need(slots, "slots", torch.int32, 1)
+        if cache.shape[2] != rank + rot or slots.shape[0] != T:
+            raise KernelError(f"latent_prepare: cache rows of {cache.shape[2]} entries, expected {rank + rot}")
+    _call("lc_latent_prepare", _ptr(proj), _dt(proj), proj.shape[1], T, heads, dim, rot, rank, _ptr(norm_weight),
+          float(eps), _ptr(positions), _ptr(rope_table), rd, 1 if pairing == "interleaved" else 0,
+          _ptr(cache if slots is not None else None), _ptr(slots), _ptr(qa), _stream())
+
+
+def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req: torch.Tensor,
+                     positions: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, page_size: int,
+                     scale: float, window: int = 0) -> torch.Tensor:
+    """Causal attention in the latent's space: queries ``qa`` [T, heads (rank + rot)] against the cached
+    rows [c | k_r] of the token's request (``cache`` [pages, page, rank + rot], ``block_table`` [R,
+    blocks]), weights softmax(q . row * scale) over the positions j <= p (and j > p - window), result
+    the weighted sum of the rows' first ``rank`` entries -> [T, heads rank]."""
+    _need(qa, "latent_attention qa", None, 2)
+    _need(cache, "latent cache", qa.dtype, 3)
+    T = qa.shape[0]
+    if qa.shape[1] != heads * (rank + rot) or cache.shape[2] != rank + rot or cache.shape[1] != page_size:
+        raise KernelError(f"latent_attention: qa {tuple(qa.shape)} or cache {tuple(cache.shape)} do not fit "
+                          f"{heads} heads of {rank} + {rot} and pages of {page_size}")
+    _need(tok_req, "tok_req", torch.int32, 1)
+    _need(positions, "positions", torch.int32, 1)
+    _need(block_table, "block table", torch.int32, 2)
+    if tok_req.shape[0] != T or positions.shape[0] != T:
+        raise KernelError("latent_attention: one request and one position per token")
+    out = torch.empty((T, heads * rank), dtype=qa.dtype, device=qa.device)
+    _call("lc_latent_attention", _ptr(qa), _dt(qa), T, heads, rank, rot, _ptr(cache), _ptr(tok_req),
+          _ptr(positions), _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
+          _ptr(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ routed experts
+@dataclass
+class Routing:
+    """A step's routing, all on the device: ``ids`` and ``weights`` [T, top] (the chosen experts, best
+    first, and what their outputs count); the (token, choice) pairs sorted by expert: ``row_start``
+    and ``tile_start`` [E + 1], ``sorted_token`` [T top] and ``entry_row`` [T top]."""
+
+    ids: torch.Tensor
+    weights: torch.Tensor
+    row_start: torch.Tensor
+    tile_start: torch.Tensor
+    sorted_token: torch.Tensor
+    entry_row: torch.Tensor
+    experts: int
+    small_tiles: bool
+    max_tiles: int
+
+
+def moe_route(logits: torch.Tensor, top: int, renormalise: bool = True, eps: float = 1e-20) -> Routing:
+    """From the router's float32 ``logits`` [T, E]: softmax over all experts, the ``top`` largest scores of
+    every token, divided by their sum + ``eps`` where ``renormalise``, and the lists that sort the
+    (token, choice) pairs by expert for :func:`moe_experts`."""
+    _need(logits, "router logits", torch.float32, 2)
+    T, E = logits.shape
+    dev = logits.device
+    ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+    weights = torch.empty((T, top), dtype=torch.float32, device=dev)
+    _call("lc_moe_route", _ptr(logits), T, E, top, 1 if renormalise else 0, float(eps), _ptr(ids), _ptr(weights),
+          _stream())
+    small = T * top <= 16 * E       # few rows an expert: tiles of 16 rows, else of 64
+    tile = 16 if small else 64
+    lists = torch.empty((2 * (E + 1) + 2 * T * top,), dtype=torch.int32, device=dev)
+    row_start, tile_start = lists[:E + 1], lists[E + 1:2 * (E + 1)]
+    sorted_token, entry_row = lists[2 * (E + 1):2 * (E + 1) + T * top], lists[2 * (E + 1) + T * top:]
+    _call("lc_moe_lists", _ptr(ids), T, top, E, tile, _ptr(row_start), _ptr(tile_start), _ptr(sorted_token),
+          _ptr(entry_row), _stream())
+    return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, small, (T * top) // tile + E)
+
+
+def moe_experts(x: torch.Tensor, w: torch.Tensor, routing: Routing, out_dtype: torch.dtype,
+                activation: Optional[str] = None, gather: bool = False) -> torch.Tensor:
+    """One of the experts' two products over the sorted rows: sorted row m, which belongs to expert e,
+    becomes ``act(x[m] . w[e]^T)`` with ``w`` [E, N, K]; ``gather``: ``x`` has a row per token and sorted
+    row m reads its token's.  -> [T top, N]"""
+    _need(x, "moe_experts x", None, 2)
+    _need(w, "moe_experts w", None, 3)
+    E, N, K = w.shape
+    rows = routing.sorted_token.shape[0]
+    if E != routing.experts or x.shape[1] != K or (not gather and x.shape[0] != rows):
+        raise KernelError(f"moe_experts: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit the routing")
+    out = torch.empty((rows, N), dtype=out_dtype, device=x.device)
+    if rows:
+        _call("lc_gemm_grouped", _ptr(x), _dt(x), K, 0, _ptr(w), _dt(w), _ptr(out), _dt(out), N, 0, rows, N, K, E,
+              _ptr(routing.sorted_token if gather else None), _ptr(routing.row_start), _ptr(routing.tile_start),
+              routing.max_tiles, 1 if routing.small_tiles else 0, ACTIVATIONS[activation] if activation else 0,
+              None, 0, 0, _stream())
+    return out
+
+
+def moe_combine(y: torch.Tensor, routing: Routing, out_dtype: torch.dtype) -> torch.Tensor:
+    """``out[t] = sum_k weights[t, k] * y[row of token t's k-th choice]`` from float32 ``y`` [T top, n]."""
+    _need(y, "moe_combine y", torch.float32, 2)
+    T, top = routing.ids.shape
+    if y.shape[0] != T * top:
+        raise KernelError(f"moe_combine: {y.shape[0]} rows for {T} tokens of {top} choices")
+    out = torch.empty((T, y.shape[1]), dtype=out_dtype, device=y.device)
+    _call("lc_moe_combine", _ptr(y), _ptr(routing.weights), _ptr(routing.entry_row), T, top, y.shape[1], _ptr(out),
+          _dt(out), _stream())
     return out
 
 

@@ -16,7 +16,7 @@ from typing import Callable, Dict, List, Optional
 
 import torch
 
-from ..config.registry import BLOCKS, EMBEDDINGS, FAMILIES, HEADS, NORMS
+from ..config.registry import BLOCKS, EMBEDDINGS, FAMILIES, HEADS, NORMS, STREAM_STEPS
 from ..config.specs import LayerSpec, ModelSpec, PartSpec
 from ..engine.batch import SiteView, StepBatch
 from ..parts import BuildContext, ResidualStream, build_part
@@ -96,6 +96,12 @@ def declared_tensors(spec: ModelSpec) -> Dict[str, ParamDecl]:
         out[spec.embedding_name] = decl
     for layer in spec.layers:
         out.update(_LayerParts(layer).declared())
+    for i, entry in enumerate(spec.run_order):
+        if entry.before is not None:
+            for logical, decl in build_part(STREAM_STEPS, entry.before).declare().items():
+                if logical not in (entry.before_names or {}):
+                    raise KeyError(f"run_order[{i}]: the stream step's tensor '{logical}' has no checkpoint name")
+                out[entry.before_names[logical]] = decl     # sites may share a tensor (a row each)
     norm = build_part(NORMS, spec.final_norm)
     for logical, decl in norm.declare().items():
         out[spec.final_norm_names[logical]] = decl
@@ -130,6 +136,13 @@ class CausalLM:
             layer = _LayerParts(layer_spec)
             layer.bind(tensors, self.ctx)
             self.layers.append(layer)
+        # what is done to the stream right before a site's layer, by site (mostly nothing)
+        self.before: Dict[int, object] = {}
+        for index, entry in enumerate(spec.run_order):
+            if entry.before is not None:
+                step = build_part(STREAM_STEPS, entry.before)
+                step.bind({logical: tensors[entry.before_names[logical]] for logical in step.declare()}, self.ctx)
+                self.before[index] = step
         self.final_norm = build_part(NORMS, spec.final_norm)
         self.final_norm.bind({logical: tensors[name]
                               for logical, name in spec.final_norm_names.items()}, self.ctx)
@@ -147,6 +160,7 @@ class CausalLM:
         for layer in self.layers:
             for _, part in layer.parts():
                 yield part
+        yield from self.before.values()
 
     # ------------------------------------------------------------------ cache needs
     def site_needs(self) -> List[Optional[object]]:
@@ -200,6 +214,8 @@ class CausalLM:
         """Run the batch's tokens through every site; float32 logits [wanted, vocab]."""
         stream = ResidualStream(self.embed.forward(batch.token_ids))
         for index, entry in enumerate(self.spec.run_order):
+            if index in self.before:
+                self.before[index].forward(stream)
             self.layers[entry.layer].block.forward(stream, sites[index])
         if batch.num_wanted == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.ctx.device)

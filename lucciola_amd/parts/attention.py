@@ -43,6 +43,9 @@ class Attention(Part):
         self.q_norm = build_part(NORMS, qk_norm) if qk_norm else None
         self.k_norm = build_part(NORMS, qk_norm) if qk_norm else None
         self.position = build_part(POSITION_ENCODINGS, position) if position else None
+        if getattr(self.position, "pairing", "half") != "half":
+            raise ValueError("attention: its kernels rotate entry i with entry i + rot/2 only "
+                             "(pairing 'half')")
 
     def declare(self) -> Dict[str, ParamDecl]:
         out = {"q_proj": ParamDecl((self.nh * self.d, self.H)),

@@ -32,3 +32,17 @@ class PreNormResidualBlock:
         stream.pending = self.mixer.forward(x, site)
         x = self._normed(self.feed_forward_norm, self.feed_forward, stream)
         stream.pending = self.feed_forward.forward(x)
+
+
+@BLOCKS.register("prenorm_mixer")
+class PreNormMixerBlock:
+    """A layer without a feed-forward: h = h + mixer(norm(h))."""
+
+    slots = {"mixer": "mixer", "mixer_norm": "norm"}
+
+    def __init__(self, mixer, mixer_norm):
+        self.mixer, self.mixer_norm = mixer, mixer_norm
+
+    def forward(self, stream: ResidualStream, site) -> None:
+        x = PreNormResidualBlock._normed(self.mixer_norm, self.mixer, stream)
+        stream.pending = self.mixer.forward(x, site)

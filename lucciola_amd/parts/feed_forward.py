@@ -57,3 +57,76 @@ class GatedMLP(Part):
         else:
             z = ops.swiglu(ops.gemm(x, self.gate_up, self.dtype))
         return ops.gemm(z, self.down, self.dtype, defer=True)
+
+
+@FEED_FORWARDS.register("mlp")
+class MLP(Part):
+    """The plain two-matrix feed-forward ``down(act(up(x)))``, no biases.  ``activation``:
+    "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or "relu_squared"."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
+        super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size,
+                         activation=activation)
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"mlp: activation '{activation}' has no kernel ({', '.join(ops.ACTIVATIONS)})")
+        self.H, self.I, self.activation = int(hidden_size), int(intermediate_size), activation
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        return {"up": ParamDecl((self.I, self.H)), "down": ParamDecl((self.H, self.I))}
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.up, self.down = tensors["up"], tensors["down"]
+        self.dtype = ctx.dtype
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        z = ops.gemm_act(x, self.up, self.activation, self.dtype)
+        return ops.gemm(z, self.down, self.dtype, defer=True)
+
+
+@FEED_FORWARDS.register("routed_mlp")
+class RoutedMLP(Part):
+    """A mixture of small two-matrix feed-forwards.  The router's logits (float32) become
+    scores over all experts (``scores``: "softmax"); each token keeps its ``top`` largest, whose
+    scores, divided by their sum + ``renormalise_eps`` where ``renormalise``, weigh the experts'
+    outputs.  On the device the (token, expert) pairs are sorted by expert, and the two products
+    run once over the sorted rows, each tile of rows with its expert's matrix; nothing of it
+    passes the host."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int,
+                 activation: str = "relu_squared", scores: str = "softmax", renormalise: bool = True,
+                 renormalise_eps: float = 1e-20):
+        super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size, experts=experts,
+                         top=top, activation=activation, scores=scores, renormalise=renormalise,
+                         renormalise_eps=renormalise_eps)
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"routed_mlp: activation '{activation}' has no kernel")
+        if scores != "softmax":
+            raise ValueError(f"routed_mlp: scores '{scores}' have no kernel (softmax)")
+        if not 1 <= int(top) <= int(experts):
+            raise ValueError(f"routed_mlp: top {top} of {experts} experts")
+        self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(experts), int(top)
+        self.activation, self.renormalise, self.renormalise_eps = activation, bool(renormalise), float(renormalise_eps)
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        out = {"router": ParamDecl((self.E, self.H))}
+        for k in range(self.E):
+            out[f"experts.{k}.up"] = ParamDecl((self.I, self.H))
+            out[f"experts.{k}.down"] = ParamDecl((self.H, self.I))
+        return out
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.router = tensors["router"]
+        self.up = stack_rows([tensors[f"experts.{k}.up"] for k in range(self.E)]).view(self.E, self.I, self.H)
+        self.down = stack_rows([tensors[f"experts.{k}.down"] for k in range(self.E)]).view(self.E, self.H, self.I)
+        self.dtype = ctx.dtype
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        logits = ops.gemm(x, self.router, torch.float32)
+        routing = ops.moe_route(logits, self.top, self.renormalise, self.renormalise_eps)
+        hidden = ops.moe_experts(x, self.up, routing, self.dtype, activation=self.activation, gather=True)
+        y = ops.moe_experts(hidden, self.down, routing, torch.float32)
+        return ops.moe_combine(y, routing, self.dtype)

@@ -1,0 +1,106 @@
+"""Latent attention as a part: attention whose keys and values are rebuilt from a small latent
+that is all the cache keeps of a token.
+
+With h the mixer's input, H heads, per head ``dim`` unrotated and ``rot_dim`` rotated query/key
+entries, values of ``vdim`` and a latent of ``kv_rank``:
+  q = W_q h, head by head [dim | rot_dim];  W_dkv h = [c' | k_r] with c = rms(c') w_norm the
+  latent and k_r (rot_dim entries, rotated by the token's position) a key part that all heads
+  share;  per head k_h = W_uk,h c, v_h = W_uv,h c;
+  score(i, j) = (q_h,plain(i) . k_h(j) + rot(q_h,rot(i)) . rot(k_r(j))) * scale,
+  softmax over the keys j the window lets i see, o_h = sum_j p_j v_h(j);
+  the heads side by side, times sigmoid(W_g h) where the part has a gate, then W_o.
+Only [c | rot(k_r)] is cached (``PagedLatent``).  The kernels never build k_h or v_h: because
+q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c, the query is taken into the latent's space
+(one small product per head), attention runs there with one shared "key" [c | k_r] and the
+"value" c for all heads, and W_uv,h is applied to the attended latent afterwards.  A step of
+single tokens and a prompt's portion go through the same kernels, so a token's result does not
+depend on how the prompt was cut.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.specs import PagedLatent
+from ..config.registry import MIXERS, POSITION_ENCODINGS
+from ..config.specs import PartSpec
+from ..kernels import ops
+from ..weights.loader import ParamDecl
+from .base import BuildContext, Part, build_part
+from .feed_forward import stack_rows
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention(Part):
+    graph_safe = True   # launches only kernels whose arguments stay put between steps
+
+    def __init__(self, hidden_size: int, num_heads: int, dim: int, rot_dim: int, vdim: int,
+                 kv_rank: int, scale: float, eps: float, position: Optional[PartSpec] = None,
+                 window: Optional[int] = None, gate: bool = False):
+        super().__init__(hidden_size=hidden_size, num_heads=num_heads, dim=dim, rot_dim=rot_dim,
+                         vdim=vdim, kv_rank=kv_rank, scale=scale, eps=eps, position=position,
+                         window=window, gate=gate)
+        self.W, self.H = int(hidden_size), int(num_heads)
+        self.dim, self.rot, self.vdim, self.rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.window = int(window) if window else None
+        self.gate = bool(gate)
+        self.position = build_part(POSITION_ENCODINGS, position) if position and self.rot else None
+        if self.position is not None and self.position.rotary_dim > self.rot:
+            raise ValueError(f"latent_attention: {self.position.rotary_dim} rotated entries in a "
+                             f"part of {self.rot}")
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        out = {"q": ParamDecl((self.H * (self.dim + self.rot), self.W)),
+               "dkv": ParamDecl((self.rank + self.rot, self.W)),
+               "dkv_norm": ParamDecl((self.rank,), role="vector", init="ones_plus_normal"),
+               "uk": ParamDecl((self.H * self.dim, self.rank)),
+               "uv": ParamDecl((self.H * self.vdim, self.rank)),
+               "o": ParamDecl((self.W, self.H * self.vdim))}
+        if self.gate:
+            out["g"] = ParamDecl((self.H * self.vdim, self.W))
+        return out
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        # one product for everything that reads the mixer's input: [q | dkv | g]
+        first = [tensors["q"], tensors["dkv"]] + ([tensors["g"]] if self.gate else [])
+        self.qdg = stack_rows(first)
+        self.norm_weight = tensors["dkv_norm"]
+        # W_uk,h transposed: the matrix that takes a head's plain query into the latent's space
+        self.uk_t = tensors["uk"].view(self.H, self.dim, self.rank).transpose(1, 2).contiguous()
+        self.uv = tensors["uv"].view(self.H, self.vdim, self.rank).contiguous()
+        self.o = tensors["o"]
+        self.dtype = ctx.dtype
+        if self.position is not None:
+            self.position.bind({}, ctx)
+
+    def cache_need(self):
+        return PagedLatent(self.rank + self.rot, self.window)
+
+    def tables_epoch(self) -> int:
+        return self.position.tables_epoch() if self.position is not None else 0
+
+    def ready(self, position: int) -> bool:
+        return self.position.ready(position) if self.position is not None else True
+
+    def forward(self, x: torch.Tensor, site) -> torch.Tensor:
+        H, dim, rot, rank, vdim = self.H, self.dim, self.rot, self.rank, self.vdim
+        batch, pages = site.batch, site.pages
+        qdg = ops.gemm(x, self.qdg, self.dtype)
+        T = qdg.shape[0]
+        q_cols = H * (dim + rot)
+        table = self.position.rotary_table(batch.max_position) if self.position is not None else None
+        pairing = self.position.pairing if self.position is not None else "half"
+        # the query in the latent's space, head by head [W_uk^T q_plain | rot(q_rot)]
+        qa = torch.empty((T, H * (rank + rot)), dtype=self.dtype, device=qdg.device)
+        ops.latent_prepare(qdg, H, dim, rot, rank, self.norm_weight, self.eps, batch.positions, table,
+                           pairing, site.cache, pages.slots if site.writes_cache else None, qa)
+        if dim:
+            ops.grouped_gemm(ops.Strided(qdg, 0, dim + rot), self.uk_t, ops.Strided(qa, 0, rank + rot), T)
+        latent = ops.latent_attention(qa, H, rank, rot, batch.tok_req, batch.positions, pages.block_table,
+                                      site.cache, pages.page_size, self.scale, self.window or 0)
+        heads = torch.empty((T, H * vdim), dtype=self.dtype, device=qdg.device)
+        gate = ops.Strided(qdg, q_cols + rank + rot, vdim) if self.gate else None
+        ops.grouped_gemm(ops.Strided(latent, 0, rank), self.uv, ops.Strided(heads, 0, vdim), T, gate=gate)
+        return ops.gemm(heads, self.o, self.dtype, defer=True)

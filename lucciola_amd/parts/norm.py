@@ -1,4 +1,4 @@
-"""RMSNorm as a part: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the last dimension
+"""The norms.  RMSNorm as a part: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the last dimension
 (reference: src/kernels/rmsnorm.cu:56-97; eps is the literal 1e-6 there, src/qwen.cc:588, and
 a parameter here)."""
 from __future__ import annotations
@@ -48,3 +48,41 @@ class RMSNorm(Part):
 
     def fused_rms(self) -> Optional[Tuple[torch.Tensor, float]]:
         return self.weight, self.eps
+
+
+@NORMS.register("dynamic_tanh")
+class DynamicTanh(Part):
+    """``y = tanh(alpha x) w + b``: a norm that takes no mean and no variance of its row.  The
+    scalar ``alpha``, the weight and the bias are learned; everything is float32 arithmetic."""
+
+    graph_safe = True
+
+    def __init__(self, size: int):
+        super().__init__(size=size)
+        self.size = int(size)
+        self.weight = self.bias = None
+        self.alpha = 1.0
+        self.dtype = None
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal"),
+                "bias": ParamDecl((self.size,), role="vector", init="normal"),
+                "alpha": ParamDecl((), role="vector", init="ones_plus_normal")}
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.weight, self.bias = tensors["weight"], tensors["bias"]
+        self.alpha = float(tensors["alpha"].item())     # a kernel argument; read once, at load
+        self.dtype = ctx.dtype
+
+    def add_norm(self, stream: ResidualStream, scaled: bool = False):
+        x = ops.dynamic_tanh(stream.h, ops.value(stream.pending), self.weight, self.bias, self.alpha,
+                             self.dtype)
+        stream.pending = None
+        return x
+
+    def add_norm_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        return ops.dynamic_tanh(stream.h, ops.value(stream.pending), self.weight, self.bias, self.alpha,
+                                self.dtype, rows=rows)
+
+    def fused_rms(self):
+        return None

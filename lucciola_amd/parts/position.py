@@ -5,10 +5,19 @@ Half-split pairing as the reference computes it (src/kernels/rope.cu:28-60): for
 theta is the literal 1e6 in the reference (src/qwen.cc:636) and a parameter here.  The
 angles' cosines and sines are tabulated once per position (computed in float64, stored as
 float32) and the kernel looks them up; the table grows when a longer position shows up.
+
+Two things are parameters beyond the reference: which entries form a pair (``pairing``:
+"half", entry i with entry i + rot/2, or "interleaved", entry 2i with entry 2i + 1; the table is
+the same, the kernels that rotate differ) and a stretching of the frequencies for contexts
+longer than the one trained on (``scaling``, the YaRN rule: with dim(t) = rot ln(original /
+(2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot - 1) and
+ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i becomes f_i / factor * ramp_i +
+f_i (1 - ramp_i), and cosines and sines are multiplied by 0.1 ln(factor) + 1).
 """
 from __future__ import annotations
 
-from typing import Optional
+import math
+from typing import Any, Dict, Optional
 
 import torch
 
@@ -28,18 +37,26 @@ class _SharedTable:
 
 @POSITION_ENCODINGS.register("rotary")
 class Rotary(Part):
-    def __init__(self, rotary_dim: int, theta: float, max_positions: int = 0):
-        super().__init__(rotary_dim=rotary_dim, theta=theta, max_positions=max_positions)
+    def __init__(self, rotary_dim: int, theta: float, max_positions: int = 0, pairing: str = "half",
+                 scaling: Optional[Dict[str, Any]] = None):
+        super().__init__(rotary_dim=rotary_dim, theta=theta, max_positions=max_positions,
+                         pairing=pairing, scaling=scaling)
         if rotary_dim % 2:
             raise ValueError(f"rotary: the rotated size {rotary_dim} must be even")
-        self.rotary_dim, self.theta = int(rotary_dim), float(theta)
+        if pairing not in ("half", "interleaved"):
+            raise ValueError(f"rotary: pairing '{pairing}' is neither 'half' nor 'interleaved'")
+        self.rotary_dim, self.theta, self.pairing = int(rotary_dim), float(theta), pairing
+        self.scaling = None
+        if scaling:
+            self.scaling = tuple(float(scaling[k]) for k in ("factor", "original", "fast", "slow"))
         self.initial = int(max_positions)
         self._shared = _SharedTable()
         self._device = None
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self._device = ctx.device
-        self._shared = ctx.shared.setdefault(("rotary table", self.rotary_dim, self.theta), _SharedTable())
+        self._shared = ctx.shared.setdefault(("rotary table", self.rotary_dim, self.theta, self.scaling),
+                                             _SharedTable())
 
     def tables_epoch(self) -> int:
         return self._shared.generation
@@ -56,8 +73,20 @@ class Rotary(Part):
         i = torch.arange(half, dtype=torch.float64)
         inv_freq = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64),
                                    2.0 * i / self.rotary_dim)
+        magnitude = 1.0
+        if self.scaling is not None:
+            factor, original, fast, slow = self.scaling
+
+            def turn_dim(turns: float) -> float:
+                return self.rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+            lo = max(math.floor(turn_dim(fast)), 0)
+            hi = min(math.ceil(turn_dim(slow)), self.rotary_dim - 1)
+            ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            inv_freq = inv_freq / factor * ramp + inv_freq * (1.0 - ramp)
+            magnitude = 0.1 * math.log(factor) + 1.0
         angle = torch.arange(count, dtype=torch.float64)[:, None] * inv_freq[None, :]
-        table = torch.cat([torch.cos(angle), torch.sin(angle)], dim=1).to(torch.float32)
+        table = (torch.cat([torch.cos(angle), torch.sin(angle)], dim=1) * magnitude).to(torch.float32)
         return table.contiguous().to(self._device)
 
     def rotary_table(self, max_position: int) -> torch.Tensor:

@@ -5,6 +5,8 @@ its function here, and CPU tests put these in place of the kernels to exercise t
 function, the cache and the scheduler without a GPU.  Nothing under ``lucciola_amd`` imports
 this file.
 """
+import math
+
 import torch
 
 F64 = torch.float64
@@ -119,6 +121,143 @@ def sample(logits, temperature=None, uniform=None):
     return out
 
 
+# ------------------------------------------------------------------ the kernels of later parts
+def dynamic_tanh(h, delta, weight, bias, alpha, out_dtype, rows=None):
+    if rows is None:
+        if delta is not None:
+            h += delta.to(torch.float32)
+        v = h.to(F64)
+    else:
+        v = h[rows.long()].to(F64)
+        if delta is not None:
+            v = (h[rows.long()] + delta[rows.long()].to(torch.float32)).to(F64)
+    return (torch.tanh(alpha * v) * weight.to(F64) + bias.to(F64)).to(out_dtype)
+
+
+def stream_add(h, delta, vector):
+    if delta is not None:
+        h += delta.to(torch.float32)
+    h += vector
+
+
+def _act(z, kind):
+    if kind == "gelu_tanh":
+        return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
+    if kind == "relu_squared":
+        return torch.clamp(z, min=0) ** 2
+    raise ValueError(kind)
+
+
+def activation(x, kind):
+    x.copy_(_act(x.to(F64), kind).to(x.dtype))
+    return x
+
+
+def gemm_act(x, w, kind, out_dtype):
+    return _act(x.to(F64) @ w.to(F64).T, kind).to(out_dtype)
+
+
+def grouped_gemm(x, w, out, rows, gate=None, activation=None):
+    G, N, K = w.shape
+    for g in range(G):
+        xs = x.tensor[:rows, x.column + g * x.group: x.column + g * x.group + K].to(F64)
+        y = xs @ w[g].to(F64).T
+        if activation:
+            y = _act(y, activation)
+        if gate is not None:
+            y = y * torch.sigmoid(gate.tensor[:rows, gate.column + g * gate.group: gate.column + g * gate.group + N].to(F64))
+        out.tensor[:rows, out.column + g * out.group: out.column + g * out.group + N] = y.to(out.tensor.dtype)
+
+
+def _turn(part, cs, rd, pairing):
+    """part [T, ..., n] (float64), cs [T, rd] cosines then sines"""
+    if cs is None or rd == 0:
+        return part
+    half = rd // 2
+    shape = [part.shape[0]] + [1] * (part.dim() - 2) + [half]
+    cos, sin = cs[:, :half].view(shape), cs[:, half:].view(shape)
+    out = part.clone()
+    if pairing == "interleaved":
+        u, v = part[..., 0:rd:2], part[..., 1:rd:2]
+        out[..., 0:rd:2] = u * cos - v * sin
+        out[..., 1:rd:2] = v * cos + u * sin
+    else:
+        u, v = part[..., :half], part[..., half:rd]
+        out[..., :half] = u * cos - v * sin
+        out[..., half:rd] = v * cos + u * sin
+    return out
+
+
+def latent_prepare(proj, heads, dim, rot, rank, norm_weight, eps, positions, rope_table, pairing, cache, slots, qa):
+    T = proj.shape[0]
+    q = proj[:, :heads * (dim + rot)].view(T, heads, dim + rot).to(F64)
+    down = proj[:, heads * (dim + rot): heads * (dim + rot) + rank + rot].to(F64)
+    c = down[:, :rank]
+    c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * norm_weight.to(F64)
+    cs = rope_table[positions.long()].to(F64) if rope_table is not None and rot else None
+    rd = rope_table.shape[1] if cs is not None else 0
+    kr = _turn(down[:, rank:], cs, rd, pairing)
+    qr = _turn(q[..., dim:], cs, rd, pairing)
+    qa.view(T, heads, rank + rot)[..., rank:] = qr.to(qa.dtype)
+    if slots is not None:
+        page = cache.shape[1]
+        row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+        for t in range(T):
+            s = int(slots[t])
+            if s >= 0:
+                cache[s // page, s % page] = row[t]
+
+
+def latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page_size, scale, window=0):
+    T = qa.shape[0]
+    q = qa.view(T, heads, rank + rot).to(F64)
+    out = torch.zeros(T, heads, rank, dtype=F64, device=qa.device)
+    reqs, pos, tables = tok_req.tolist(), positions.tolist(), block_table.tolist()
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - window + 1) if window else 0
+        table = tables[reqs[t]]
+        js = list(range(lo, p + 1))
+        pages = torch.tensor([table[j // page_size] for j in js], dtype=torch.long)
+        assert (pages >= 0).all(), "latent attention reads a page that was given back"
+        offs = torch.tensor([j % page_size for j in js], dtype=torch.long)
+        rows = cache[pages, offs].to(F64)                  # [n, rank + rot]
+        w = torch.softmax((q[t] @ rows.T) * scale, dim=-1)  # [heads, n]
+        out[t] = w @ rows[:, :rank]
+    return out.reshape(T, heads * rank).to(qa.dtype)
+
+
+class _Routing:
+    pass
+
+
+def moe_route(logits, top, renormalise=True, eps=1e-20):
+    s = torch.softmax(logits.to(F64), dim=-1)
+    picked, ids = torch.topk(s, top, dim=-1)
+    if renormalise:
+        picked = picked / (picked.sum(-1, keepdim=True) + eps)
+    r = _Routing()
+    r.ids, r.weights = ids.to(torch.int32), picked.to(torch.float32)
+    return r
+
+
+def moe_experts(x, w, routing, out_dtype, activation=None, gather=False):
+    """Rows in (token, choice) order here: the order of the sorted rows is the kernels' own matter."""
+    T, top = routing.ids.shape
+    out = torch.zeros(T * top, w.shape[1], dtype=F64, device=x.device)
+    for t in range(T):
+        for k in range(top):
+            row = x[t] if gather else x[t * top + k]
+            y = w[int(routing.ids[t, k])].to(F64) @ row.to(F64)
+            out[t * top + k] = _act(y, activation) if activation else y
+    return out.to(out_dtype)
+
+
+def moe_combine(y, routing, out_dtype):
+    T, top = routing.ids.shape
+    return (y.to(F64).view(T, top, -1) * routing.weights.to(F64)[:, :, None]).sum(1).to(out_dtype)
+
+
 def attention_takes_shares(*args, **kwargs):
     return False
 
@@ -129,7 +268,8 @@ def feed_tokens(ids, source, sampled):
 
 
 ALL = ("feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
-       "swiglu", "sample")
+       "swiglu", "sample", "dynamic_tanh", "stream_add", "activation", "gemm_act", "grouped_gemm",
+       "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine")
 
 
 def install(monkeypatch):

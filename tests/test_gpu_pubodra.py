@@ -1,0 +1,186 @@
+"""The Pubodra design on the GPU: every kernel it brought against the plain torch version of the
+same operation, and the engine against the plain whole-sequence implementation
+(``plain_pubodra``) in the four families of traces, in float32 and in bfloat16."""
+import pytest
+import torch
+
+import plain_pubodra
+import pubodra_configs
+import reference_ops
+import traces
+from helpers import compare, make_runner, prompts_for, random_weights, replay
+from lucciola_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+LENGTHS = {"A": [5, 1, 47, 90, 130], "B": [2, 61, 33, 100], "C": [150, 9, 230, 70]}
+_cache = {}
+
+
+def case(key):
+    if key not in _cache:
+        cfg, page, seed = pubodra_configs.ALL[key]
+        weights = random_weights(cfg, seed, std=pubodra_configs.STD)
+        prompts = prompts_for({"vocab_size": cfg["vocab"]}, LENGTHS[key], seed)
+        refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+        _cache[key] = (cfg, page, weights, prompts, refs)
+    return _cache[key]
+
+
+def close(got, want, dtype, what):
+    tol = 3e-6 if dtype == torch.float32 else 1.2e-2
+    err = float((got.double() - want.double()).abs().max() / want.double().abs().max().clamp_min(1e-9))
+    assert err < tol, f"{what}: relative error {err:.3e}"
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,rows", [(50, None), (192, None), (1030, [3, 0, 3])])
+def test_dynamic_tanh(dtype, n, rows):
+    g = torch.Generator().manual_seed(n)
+    h = torch.randn(5, n, generator=g) * 3
+    delta = torch.randn(5, n, generator=g).to(dtype)
+    w, b = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    idx = torch.tensor(rows, dtype=torch.int32) if rows else None
+    h_ref = h.clone()
+    want = reference_ops.dynamic_tanh(h_ref, delta, w, b, 0.7, dtype, idx)
+    h_dev = h.to(DEV)
+    got = ops.dynamic_tanh(h_dev, delta.to(DEV), w.to(DEV), b.to(DEV), 0.7, dtype, idx.to(DEV) if rows else None)
+    close(got.cpu(), want, dtype, "dynamic tanh")
+    assert torch.equal(h_dev.cpu(), h_ref), "the stream after the addition"
+
+
+def test_stream_add_and_activations():
+    g = torch.Generator().manual_seed(1)
+    h, delta, vec = torch.randn(7, 33, generator=g), torch.randn(7, 33, generator=g).bfloat16(), torch.randn(33, generator=g)
+    want = h.clone()
+    reference_ops.stream_add(want, delta, vec)
+    got = h.to(DEV)
+    ops.stream_add(got, delta.to(DEV), vec.to(DEV))
+    assert torch.allclose(got.cpu(), want, atol=1e-6)
+    for kind in ops.ACTIVATIONS:
+        for dtype in (torch.float32, torch.bfloat16):
+            x = (torch.randn(11, 37, generator=g) * 3).to(dtype)
+            want = reference_ops.activation(x.clone(), kind)
+            close(ops.activation(x.to(DEV), kind).cpu(), want, dtype, kind)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,G,N,K", [(1, 3, 21, 7), (16, 2, 64, 32), (77, 5, 18, 300), (130, 1, 100, 9)])
+def test_grouped_product_over_heads(dtype, rows, G, N, K):
+    g = torch.Generator().manual_seed(rows * 7 + G)
+    pad_x, pad_o = 5, 3
+    x = torch.randn(rows, pad_x + G * (K + 2), generator=g).to(dtype)
+    w = torch.randn(G, N, K, generator=g).bfloat16()
+    gate = torch.randn(rows, G * N + 4, generator=g).to(dtype)
+    for use_gate, act in ((False, None), (True, None), (False, "relu_squared")):
+        out_ref = torch.zeros(rows, pad_o + G * N, dtype=dtype)
+        out_dev = torch.zeros(rows, pad_o + G * N, dtype=dtype, device=DEV)
+        gate_ref = ops.Strided(gate, 4, N) if use_gate else None
+        gate_dev = ops.Strided(gate.to(DEV), 4, N) if use_gate else None
+        reference_ops.grouped_gemm(ops.Strided(x, pad_x, K + 2), w, ops.Strided(out_ref, pad_o, N), rows, gate_ref, act)
+        ops.grouped_gemm(ops.Strided(x.to(DEV), pad_x, K + 2), w.to(DEV), ops.Strided(out_dev, pad_o, N), rows, gate_dev, act)
+        close(out_dev.cpu(), out_ref, dtype, f"grouped product gate={use_gate} act={act}")
+        assert float(out_dev[:, :pad_o].abs().max()) == 0.0, "columns before the first group were written"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,top,H,I", [(1, 4, 4, 20, 12), (9, 5, 1, 33, 17), (70, 12, 3, 64, 40), (300, 3, 2, 48, 64)])
+def test_routed_experts(dtype, T, E, top, H, I):
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    logits = torch.randn(T, E, generator=g) * 2
+    up, down = (torch.randn(E, I, H, generator=g) * 0.2).bfloat16(), (torch.randn(E, H, I, generator=g) * 0.2).bfloat16()
+    r_ref = reference_ops.moe_route(logits, top, True, 1e-20)
+    want = reference_ops.moe_combine(
+        reference_ops.moe_experts(reference_ops.moe_experts(x, up, r_ref, dtype, "relu_squared", True), down, r_ref,
+                                  torch.float32), r_ref, dtype)
+    r = ops.moe_route(logits.to(DEV), top, True, 1e-20)
+    assert torch.equal(r.ids.cpu(), r_ref.ids), "chosen experts"
+    assert torch.allclose(r.weights.cpu(), r_ref.weights, atol=1e-6)
+    starts = r.row_start.cpu().tolist()
+    assert starts[0] == 0 and starts[-1] == T * top and starts == sorted(starts)
+    hidden = ops.moe_experts(x.to(DEV), up.to(DEV), r, dtype, activation="relu_squared", gather=True)
+    got = ops.moe_combine(ops.moe_experts(hidden, down.to(DEV), r, torch.float32), r, dtype)
+    close(got.cpu(), want, dtype, "routed experts")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,dim,rot,rank,rd,pairing,page,window",
+                         [(3, 7, 10, 21, 6, "interleaved", 8, 17), (4, 16, 8, 32, 8, "interleaved", 4, 0),
+                          (5, 0, 12, 40, 12, "half", 16, 70), (1, 5, 0, 9, 0, "interleaved", 2, 3),
+                          (9, 8, 16, 300, 16, "interleaved", 16, 130)])
+def test_latent_attention_kernels(dtype, heads, dim, rot, rank, rd, pairing, page, window):
+    """Two requests of unequal length written to scattered pages in two portions each, then read."""
+    g = torch.Generator().manual_seed(heads * 100 + rank)
+    lengths, pages = [150, 37], 40
+    width = heads * (dim + rot) + rank + rot + 3
+    caches = [torch.zeros(pages, page, rank + rot, dtype=dtype), torch.zeros(pages, page, rank + rot, dtype=dtype, device=DEV)]
+    table = torch.randn(200, rd, generator=g) if rd else None
+    w = torch.rand(rank, generator=g) + 0.5
+    order = torch.randperm(pages, generator=g).tolist()
+    per = -(-max(lengths) // page)
+    block_table = torch.full((2, per), -1, dtype=torch.int32)
+    for r, n in enumerate(lengths):
+        for b in range(-(-n // page)):
+            block_table[r, b] = order.pop()
+    done = [0, 0]
+    for cut in (0.6, 1.0):
+        tok_req, positions = [], []
+        for r, n in enumerate(lengths):
+            upto = int(n * cut)
+            tok_req += [r] * (upto - done[r])
+            positions += list(range(done[r], upto))
+            done[r] = upto
+        T = len(tok_req)
+        tok_req, positions = torch.tensor(tok_req, dtype=torch.int32), torch.tensor(positions, dtype=torch.int32)
+        slots = (block_table[tok_req.long(), (positions // page).long()] * page + positions % page).to(torch.int32)
+        proj = torch.randn(T, width, generator=g).to(dtype)
+        latent_q = torch.randn(T, heads, rank, generator=g).to(dtype)     # what the product per head would fill in
+        outs = []
+        for where, cache in zip(("cpu", DEV), caches):
+            o = reference_ops if where == "cpu" else ops
+            qa = torch.zeros(T, heads * (rank + rot), dtype=dtype, device=where)
+            o.latent_prepare(proj.to(where), heads, dim, rot, rank, w.to(where), 1e-5, positions.to(where),
+                             table.to(where) if rd else None, pairing, cache, slots.to(where), qa)
+            qa.view(T, heads, rank + rot)[..., :rank] = latent_q.to(where)
+            outs.append((qa.cpu(), o.latent_attention(qa, heads, rank, rot, tok_req.to(where), positions.to(where),
+                                                      block_table.to(where), cache, page, 0.3, window).cpu()))
+        close(outs[1][0], outs[0][0], dtype, "rotated queries")
+        close(caches[1].cpu(), caches[0], dtype, "cache rows")
+        caches[1].copy_(caches[0])        # the same rows on both sides for the attention itself
+        close(outs[1][1], outs[0][1], dtype, "latent attention")
+
+
+def test_rotary_table_stretched():
+    """The part's table against the plain implementation's frequencies."""
+    from lucciola_amd.parts.position import Rotary
+    from lucciola_amd.parts.base import BuildContext
+    scaling = {"factor": 8.0, "original": 64, "fast": 16.0, "slow": 2.0}
+    part = Rotary(12, 5000.0, pairing="interleaved", scaling=scaling)
+    part.bind({}, BuildContext(torch.float32, torch.device(DEV)))
+    table = part.rotary_table(300).cpu().double()
+    f, mag = plain_pubodra.rotary_frequencies(12, 5000.0, scaling)
+    angle = torch.arange(table.shape[0], dtype=torch.float64)[:, None] * f[None, :]
+    assert torch.allclose(table[:, :6], torch.cos(angle) * mag, atol=1e-6)
+    assert torch.allclose(table[:, 6:], torch.sin(angle) * mag, atol=1e-6)
+
+
+# ------------------------------------------------------------------ the engine
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
+def test_replay_families(dtype, key, family):
+    cfg, page, weights, prompts, refs = case(key)
+    steps = {"whole": traces.whole, "tail": traces.tail_decode, "chunked": traces.chunked,
+             "mixed": traces.mixed}[family](prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    got = replay(runner, steps)
+    assert len(got) == sum(len(p) for p in prompts.values())
+    worst = compare(got, cfg, weights, prompts, TOL[dtype], refs)
+    print(f"{key} {family} {dtype}: worst relative error {worst:.3e}")
+    assert not runner.cache.requests
+    for g in runner.cache.groups:
+        assert g.pool.num_free() == blocks
