@@ -329,6 +329,135 @@ def mixed_workload(dtype, dev, block_size, run_ahead, new_tokens, max_tokens_per
     return out
 
 
+# ---------------------------------------------------------------------------------------------
+# Two designs side by side (--workload designs): the Pubodra decoder (latent attention with a
+# window and an output gate, Dynamic Tanh norms, a dense or a routed feed-forward) beside the
+# Qwen3 decoder at equal width, heads, head size, feed-forward width, vocabulary and depth.
+DESIGN_SIZES = {
+    # name: width, heads, feed-forward width
+    "w2048": (2048, 16, 8192),
+    "w4096": (4096, 32, 12288),
+}
+DESIGN_VOCAB = 32768
+DESIGN_LAYERS = 4
+
+
+def design_configs(name, routed):
+    width, heads, ff = DESIGN_SIZES[name]
+    qwen = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=DESIGN_LAYERS, hidden_size=width,
+                num_attention_heads=heads, num_key_value_heads=max(1, heads // 4), head_dim=128,
+                intermediate_size=ff, vocab_size=DESIGN_VOCAB, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=True, max_position_embeddings=40960, initializer_range=0.02)
+    mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+             "mask": {"size": 4096},
+             "rot": {"base": 1000000.0, "dims": 64,
+                     "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    dense = {"kind": "dense", "ff": ff}
+    # the routed layer moves as many weights per token as the dense one: 4 of 32 experts of ff / 4
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}}
+    pubodra = {"architecture": "Pubodra", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+               "initializer_range": 0.02,
+               "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": moe if routed and i % 2 else dense}
+                          for i in range(DESIGN_LAYERS)]}
+    return qwen, pubodra
+
+
+def design_run(cfg, dtype, dev, block_size, prompt, batches, context, steps):
+    """Prompt and decode throughput of one configuration through the runner's own step."""
+    import torch
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.engine.batch import StepEntry
+    from lucciola_amd.engine.loading import random_model
+    from lucciola_amd.engine.runner import ModelRunner
+    from lucciola_amd.sampling.sampler import Sampler, SamplingParams
+
+    model, _ = random_model(cfg, seed=0, dtype=dtype, device=dev)
+    most = max(batches)
+    blocks = most * (-(-(context + steps + 8) // block_size)) + (-(-prompt // block_size)) + 8
+    runner = ModelRunner(model, EngineConfig(dtype=dtype, block_size=block_size, max_blocks=blocks,
+                                             max_seqs=most + 2, device=dev))
+    for stored in runner.cache.storage.values():
+        for need in stored:
+            for t in (need if isinstance(need, (tuple, list)) else (need,)):
+                t.normal_(0, 0.5)
+    sampler = Sampler()
+    vocab = model.vocab_size
+    gen = torch.Generator().manual_seed(5)
+    out = {}
+    best = None
+    for r in range(3):
+        ids = torch.randint(0, vocab, (prompt,), generator=gen).tolist()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        logits = runner.step([StepEntry(f"p{r}", ids, [prompt - 1])])
+        sampler.sample(logits, [SamplingParams()], [0])
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t) * 1e3
+        runner.finish(f"p{r}")
+        if r > 0:
+            best = ms if best is None else min(best, ms)
+    out[f"prefill_{prompt}"] = {"ms": round(best, 3), "tokens_per_s": round(prompt / (best / 1e3), 1)}
+    for batch in batches:
+        names = [f"d{batch}_{i}" for i in range(batch)]
+        for n in names:
+            runner.cache.admit(n)
+            runner.cache.reserve(n, context - 1)
+            runner.cache.commit(n)
+        tokens = torch.randint(0, vocab, (batch,), generator=gen).tolist()
+        params = [SamplingParams(max_new_tokens=1 << 30)] * batch
+
+        def one():
+            nonlocal tokens
+            logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, tokens)])
+            tokens = sampler.sample(logits, params, [0] * batch)
+        for _ in range(4):
+            one()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t) * 1e3 / steps
+        for n in names:
+            runner.finish(n)
+        out[f"decode_b{batch}_ctx{context}"] = {"ms": round(ms, 4), "tokens_per_s": round(batch / (ms / 1e3), 1)}
+    del runner, model
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def designs_workload(args, dev):
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    batches = [int(b) for b in args.design_batches.split(",") if b]
+    results = {}
+    for name in [n for n in args.design_sizes.split(",") if n]:
+        for routed in (False, True):
+            qwen, pubodra = design_configs(name, routed)
+            if not routed:
+                results[f"{name}/qwen3"] = design_run(qwen, dtype, dev, args.block_size, args.prefill_tokens,
+                                                      batches, args.design_context, args.steps)
+                say(f"{name} qwen3: {results[f'{name}/qwen3']}")
+            key = f"{name}/pubodra_{'routed' if routed else 'dense'}"
+            results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
+                                      args.design_context, args.steps)
+            say(f"{key}: {results[key]}")
+    first = next(iter(results))
+    head = f"decode_b{batches[0]}_ctx{args.design_context}"
+    key = [k for k in results if "pubodra_dense" in k][0]
+    line = {"metric": f"decode tok/s (Pubodra-shaped, {key.split('/')[0]}, {DESIGN_LAYERS} layers, batch {batches[0]}, "
+                      f"context {args.design_context})",
+            "value": results[key][head]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": 4, "ms_per_step": results[key][head]["ms"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": args.dtype, "data": "synthetic: random weights, random token ids, "
+            "cache of the live requests filled with random rows",
+            "config": {"layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "sizes": {n: DESIGN_SIZES[n] for n in DESIGN_SIZES},
+                       "page_size": args.block_size, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
+            "designs": results}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -358,7 +487,10 @@ def main() -> int:
     ap.add_argument("--others", type=int, default=-1, choices=[-1, 0, 1],
                     help="1: also run the 32B-shaped points and the 0.6B-shaped mixed workload; "
                          "-1 (default): only in the default run (8B-shaped, bf16, all layers)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+    ap.add_argument("--design-sizes", default="w2048,w4096", help="designs: which of " + ", ".join(DESIGN_SIZES))
+    ap.add_argument("--design-batches", default="8,64", help="designs: decode batch sizes")
+    ap.add_argument("--design-context", type=int, default=2048, help="designs: tokens a decoding request holds")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "designs"],
                     help="decode: the default line; mixed: only the 0.6B-shaped mixed workload, as a line of its own")
     ap.add_argument("--new-tokens", type=int, default=128, help="mixed: tokens generated per request")
     ap.add_argument("--max-tokens-per-step", type=int, default=2048, help="mixed: the scheduler's budget")
@@ -370,6 +502,8 @@ def main() -> int:
     import torch
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.workload == "designs":
+        return designs_workload(args, dev)
     if args.workload == "mixed":
         m = mixed_workload(args.dtype, dev, args.block_size, args.run_ahead, args.new_tokens, args.max_tokens_per_step)
         line = {

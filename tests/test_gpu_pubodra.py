@@ -114,7 +114,8 @@ def test_routed_experts(dtype, T, E, top, H, I):
 def test_latent_attention_kernels(dtype, heads, dim, rot, rank, rd, pairing, page, window):
     """Two requests of unequal length written to scattered pages in two portions each, then read."""
     g = torch.Generator().manual_seed(heads * 100 + rank)
-    lengths, pages = [150, 37], 40
+    lengths = [150, 37]
+    pages = sum(-(-n // page) for n in lengths) + 3
     width = heads * (dim + rot) + rank + rot + 3
     caches = [torch.zeros(pages, page, rank + rot, dtype=dtype), torch.zeros(pages, page, rank + rot, dtype=dtype, device=DEV)]
     table = torch.randn(200, rd, generator=g) if rd else None
