@@ -185,3 +185,14 @@ def forward(cfg, weights, ids, positions=None, trace=None):
         if trace is not None:
             trace.append(x.clone())
     return linear(_norm(x, weights, "final.norm"), weights["embed"])
+
+
+def greedy(cfg, weights, prompt, new_tokens):
+    """Greedy generation by running the whole sequence again for every token; ties go to the
+    lowest index."""
+    ids, out = list(prompt), []
+    for _ in range(new_tokens):
+        tok = int(torch.argmax(forward(cfg, weights, ids)[-1]))
+        out.append(tok)
+        ids.append(tok)
+    return out

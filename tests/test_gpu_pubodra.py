@@ -185,3 +185,183 @@ def test_replay_families(dtype, key, family):
     assert not runner.cache.requests
     for g in runner.cache.groups:
         assert g.pool.num_free() == blocks
+
+
+# ------------------------------------------------------------------ one mechanism a model
+def _one_layer(mixer, mlp, **more):
+    cfg = {"architecture": "Pubodra", "vocab": 97, "width": 40, "norm": {"eps": 2e-6},
+           "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp}]}
+    cfg.update(more)
+    return cfg
+
+
+MECHANISMS = {
+    "mixer alone": _one_layer(pubodra_configs._mixer(3, 8, 6, 5, 12, 0.3, 11, base=200.0), None),
+    "one head, nothing rotated": _one_layer({"heads": 1, "dim": 9, "rot_dim": 0, "vdim": 7, "kv_rank": 10, "scale": 0.4,
+                                              "mask": {"size": 5}}, None),
+    "everything rotated, no window": _one_layer(pubodra_configs._mixer(2, 0, 12, 6, 8, 0.3, None, base=50.0,
+                                                                        scaling=pubodra_configs.YARN), None),
+    "dense feed-forward": _one_layer(pubodra_configs._mixer(2, 4, 4, 4, 8, 0.5, 64), pubodra_configs._dense(33)),
+    "every expert chosen": _one_layer(pubodra_configs._mixer(2, 4, 4, 4, 8, 0.5, 64), pubodra_configs._moe(12, 4, 4)),
+    "one expert of many": _one_layer(pubodra_configs._mixer(2, 4, 4, 4, 8, 0.5, 64), pubodra_configs._moe(20, 70, 1)),
+    "a stack run once": _one_layer(pubodra_configs._mixer(2, 4, 4, 4, 8, 0.5, 3), pubodra_configs._dense(16),
+                                   loop={"start": 0, "stop": 1, "times": 1}),
+    "one layer run four times": _one_layer(pubodra_configs._mixer(2, 4, 4, 4, 8, 0.5, 7), pubodra_configs._moe(16, 3, 2),
+                                           loop={"start": 0, "stop": 1, "times": 4}),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(MECHANISMS))
+def test_each_mechanism(name, dtype):
+    """Models of one layer that have one mechanism each, with sizes of 1, of 0 and equal to one
+    another, fed whole, in portions and token by token."""
+    cfg = MECHANISMS[name]
+    weights = random_weights(cfg, 5, std=0.15 if dtype == "float32" else 0.06)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [23, 2, 58], 3)
+    refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    every_token = [([(n, [t], [0])], [n] if i == len(ids) - 1 else []) for n, ids in prompts.items()
+                   for i, t in enumerate(ids)]
+    for steps in (traces.whole(prompts), traces.chunked(prompts, sizes=(2, 9, 3, 2, 17)), every_token):
+        runner = make_runner(cfg, weights, 4, 40, dtype, DEV)
+        compare(replay(runner, steps), cfg, weights, prompts, TOL[dtype], refs)
+
+
+# ------------------------------------------------------------------ edges of the window, far keys
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,page", [(33, 16), (64, 16), (17, 4), (0, 8)])
+def test_one_key_carries_the_weight(dtype, window, page):
+    """Among 300 cached rows one row's score stands out (its latent lies along the query); it is put
+    far back, on both sides of every page border near the window's edge, just inside and just
+    outside the window, and is read by a lone token and by the last row of a portion.  Where the
+    query sees it, the result is that row's latent; where it does not, it is not."""
+    heads, rank, rot, n = 2, 16, 4, 300
+    g = torch.Generator().manual_seed(window + page)
+    pages = -(-n // page) + 2
+    order = torch.randperm(pages, generator=g).tolist()
+    block_table = torch.tensor([order[:-(-n // page)]], dtype=torch.int32)
+    base = (torch.randn(n, rank + rot, generator=g) * 0.1)
+    marker = torch.zeros(rank + rot)
+    marker[3] = 6.0
+    p = n - 1
+    edge = p - window + 1 if window else 0
+    places = sorted({0, 1, edge - 1, edge, edge + 1, p - 1, p} | {b + d for b in range(edge - page, edge + page + 1, 1)
+                                                                  if b % page == 0 for d in (-1, 0)})
+    for place in [j for j in places if 0 <= j <= p]:
+        rows = base.clone()
+        rows[place] = marker
+        cache = torch.zeros(pages, page, rank + rot, dtype=dtype)
+        for j in range(n):
+            cache[block_table[0, j // page], j % page] = rows[j].to(dtype)
+        qa = torch.zeros(heads * (rank + rot))
+        qa[3] = qa[rank + rot + 3] = 4.0
+        seen = place >= edge
+        for portion in (1, 7):
+            T = portion
+            positions = torch.arange(p - T + 1, p + 1, dtype=torch.int32)
+            q = qa.to(dtype).repeat(T, 1)
+            args = (heads, rank, rot, torch.zeros(T, dtype=torch.int32), positions, block_table)
+            want = reference_ops.latent_attention(q, *args, cache, page, 1.0, window)
+            got = ops.latent_attention(q.to(DEV), heads, rank, rot, args[3].to(DEV), positions.to(DEV),
+                                       block_table.to(DEV), cache.to(DEV), page, 1.0, window).cpu()
+            close(got, want, dtype, f"marker at {place}, window {window}, portion of {portion}")
+            last = got[-1].float().view(heads, rank)
+            assert (float(last[0, 3]) > 5.5) == seen, f"marker at {place} (edge {edge}): seen is {seen}"
+
+
+# ------------------------------------------------------------------ the engine's other ways in
+def engine_for(cfg, weights, page, blocks, dtype, **kw):
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.config.registry import architecture_for
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.engine.loading import _build
+    from lucciola_amd.weights.loader import DictSource
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), dtype, DEV)
+    return LLMEngine(model, config, EngineConfig(dtype=dtype, block_size=page, max_blocks=blocks, device=DEV, **kw))
+
+
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_greedy_generation_through_the_engine(key):
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = pubodra_configs.ALL[key]
+    weights = random_weights(cfg, seed, std=0.2)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [5, 11, 37], seed + 30).values())
+    engine = engine_for(cfg, weights, page, 64, "float32", max_tokens_per_step=16, max_seqs=4)
+    got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
+    assert got == [plain_pubodra.greedy(cfg, weights, p, 8) for p in prompts]
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "C"])
+def test_long_decoding_and_stale_pages(dtype, key):
+    """A short prompt, then 260 tokens one by one (in bfloat16 through captured steps), past every
+    window, in a cache whose pages hold the rows of other requests when they are taken."""
+    cfg, page, seed = pubodra_configs.ALL[key]
+    weights = random_weights(cfg, seed, std=pubodra_configs.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [268, 270], seed + 7)
+    refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.tail_decode(prompts, tail=260)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    for stored in runner.cache.storage.values():
+        stored[0].normal_(0, 30.0)
+    compare(replay(runner, steps), cfg, weights, prompts, TOL[dtype], refs)
+    if dtype == "bfloat16":
+        assert runner.graph_replays > 200
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from lucciola_amd.weights.random_init import write_model_folder
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = pubodra_configs.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "model"), dict(cfg, initializer_range=pubodra_configs.STD), seed)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [70, 33, 50, 3, 61], seed)
+    steps = traces.mixed(prompts, seed=3)
+    lines, index, fed = [], {}, {}
+    for i, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": i, "end": end, "entries": [{"id": n, "tokens": t, "want": w} for n, t, w in entries]}))
+        rows = []
+        for n, t, w in entries:
+            rows += [(n, fed.get(n, 0) + k) for k in w]
+            fed[n] = fed.get(n, 0) + len(t)
+        index[i] = rows
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(traces.max_live_tokens(steps, 64))],
+                          input="\n".join(lines) + "\n", text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [x for i in range(len(steps)) for x in ("done", str(i))]
+    got = {}
+    for i, rows in index.items():
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"])
+        for r, key in enumerate(rows):
+            got[key] = torch.from_numpy(data[r].astype("float64"))
+    refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    compare(got, cfg, weights, prompts, TOL[dtype], refs)
+
+
+def test_float32_logits_do_not_depend_on_the_cut():
+    """The same bits whole, in portions and token by token: every sum's order follows from the
+    token alone."""
+    cfg, page, seed = pubodra_configs.ALL["B"]
+    weights = random_weights(cfg, seed, std=pubodra_configs.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [75, 40], seed)
+    runs = []
+    for steps in (traces.whole(prompts), traces.chunked(prompts), traces.tail_decode(prompts, tail=30), traces.mixed(prompts)):
+        runs.append(replay(make_runner(cfg, weights, page, 40, "float32", DEV), steps))
+    for other in runs[1:]:
+        for key, row in runs[0].items():
+            assert torch.equal(row, other[key]), f"{key}: the bits differ between two cuts"
