@@ -93,7 +93,9 @@ class LatentAttention(Part):
         table = self.position.rotary_table(batch.max_position) if self.position is not None else None
         pairing = self.position.pairing if self.position is not None else "half"
         # the query in the latent's space, head by head [W_uk^T q_plain | rot(q_rot)]
-        qa = torch.empty((T, H * (rank + rot)), dtype=self.dtype, device=qdg.device)
+        # (without plain query entries nothing of the query reaches the latent: that part is zero)
+        make = torch.empty if dim else torch.zeros
+        qa = make((T, H * (rank + rot)), dtype=self.dtype, device=qdg.device)
         ops.latent_prepare(qdg, H, dim, rot, rank, self.norm_weight, self.eps, batch.positions, table,
                            pairing, site.cache, pages.slots if site.writes_cache else None, qa)
         if dim:
