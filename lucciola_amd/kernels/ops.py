@@ -76,6 +76,9 @@ _SIGNATURES = {
     "lc_gemm_grouped": "piqqpipiqqiiiipppiiipqqp",
     "lc_latent_prepare": "piqiiiiipfppiipppp",
     "lc_latent_attention": "piiiiippppiifipp",
+    "lc_latent_bf16_supported": "ii",
+    "lc_latent_bf16_splits": "ii",
+    "lc_latent_attention_bf16": "piiiippiipiifipippp",
     "lc_moe_max_experts": "",
     "lc_moe_route": "piiiifppp",
     "lc_moe_lists": "piiiippppp",
@@ -1017,9 +1020,42 @@ def latent_prepare(proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int
           _ptr(cache if slots is not None else None), _ptr(slots), _ptr(qa), _stream())
 
 
+class _LatentSwitch(threading.local):
+    on = True
+
+
+_latent_fast = _LatentSwitch()      # per thread, like the library's own switches
+
+
+def latent_matrix_cores(on: bool) -> bool:
+    """Whether bfloat16 latent attention may run on the matrix-core kernel (tests run both); returns
+    the setting before."""
+    before = _latent_fast.on
+    _latent_fast.on = bool(on)
+    return before
+
+
+LATENT_PLAN = "latent_attention"
+LATENT_TILE = 16                # tokens of one work item of the matrix-core latent attention kernel
+
+
+def plan_latent_attention(layout):
+    """The work list of the matrix-core latent attention kernel for one step's batch (a planner in the
+    sense of ``Part.batch_planner``): every request's tokens of this step cut into tiles of up to
+    LATENT_TILE, four numbers each (first token row, tokens, request, first position); a request
+    that brings one token is a tile of one token, which the kernel serves head by head."""
+    tiles = []
+    for r in range(layout.num_requests):
+        first, n = layout.q_start[r], layout.q_start[r + 1] - layout.q_start[r]
+        for t0 in range(0, n, LATENT_TILE):
+            tiles.append((first + t0, min(LATENT_TILE, n - t0), r, layout.first_position[r] + t0))
+    return ({"tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)},
+            {"any_portion": any(t[1] > 1 for t in tiles), "num_tiles": len(tiles)})
+
+
 def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req: torch.Tensor,
                      positions: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, page_size: int,
-                     scale: float, window: int = 0) -> torch.Tensor:
+                     scale: float, window: int = 0, plan=None, max_ctx: int = 0) -> torch.Tensor:
     """Causal attention in the latent's space: queries ``qa`` [T, heads (rank + rot)] against the cached
     rows [c | k_r] of the token's request (``cache`` [pages, page, rank + rot], ``block_table`` [R,
     blocks]), weights softmax(q . row * scale) over the positions j <= p (and j > p - window), result
@@ -1036,6 +1072,29 @@ def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req:
     if tok_req.shape[0] != T or positions.shape[0] != T:
         raise KernelError("latent_attention: one request and one position per token")
     out = torch.empty((T, heads * rank), dtype=qa.dtype, device=qa.device)
+    if T == 0:
+        return out
+    lib = library()
+    if (qa.dtype == torch.bfloat16 and plan is not None and _latent_fast.on
+            and lib.lc_latent_bf16_supported(rank, rot)):
+        # the matrix-core kernel, over the planner's tiles; few tiles: their keys are shared out
+        tiles, any_portion = plan.arrays["tiles"], plan.info["any_portion"]
+        workgroups = tiles.shape[0] * (-(-heads // 4) if any_portion else -(-heads // 64))
+        most = block_table.shape[1] * page_size if max_ctx <= 0 else max_ctx
+        splits = lib.lc_latent_bf16_splits(workgroups, min(most, window) if window > 0 else most)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty((T * heads * splits * rank,), dtype=torch.float32, device=qa.device)
+            part_ml = torch.empty((T * heads * splits * 2,), dtype=torch.float32, device=qa.device)
+        _call("lc_latent_attention_bf16", _ptr(qa), T, heads, rank, rot, _ptr(cache), _ptr(tiles), tiles.shape[0],
+              1 if any_portion else 0, _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
+              _ptr(out), splits, _ptr(part_o), _ptr(part_ml), _stream())
+        return out
+    if qa.dtype == torch.bfloat16 and plan is not None and _latent_fast.on and rank * heads >= 1024:
+        _say_once(("latent attention", rank, rot),
+                  f"bfloat16 latent attention with a latent of {rank} and {rot} rotated entries has no matrix-core "
+                  "kernel (a latent of a multiple of 16 up to 512, rows of a multiple of 8 up to 640): the general "
+                  "kernel runs, correct and many times slower")
     _call("lc_latent_attention", _ptr(qa), _dt(qa), T, heads, rank, rot, _ptr(cache), _ptr(tok_req),
           _ptr(positions), _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
           _ptr(out), _stream())

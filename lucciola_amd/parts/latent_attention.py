@@ -78,6 +78,9 @@ class LatentAttention(Part):
     def cache_need(self):
         return PagedLatent(self.rank + self.rot, self.window)
 
+    def batch_planner(self):
+        return ops.LATENT_PLAN, ops.plan_latent_attention
+
     def tables_epoch(self) -> int:
         return self.position.tables_epoch() if self.position is not None else 0
 
@@ -101,7 +104,8 @@ class LatentAttention(Part):
         if dim:
             ops.grouped_gemm(ops.Strided(qdg, 0, dim + rot), self.uk_t, ops.Strided(qa, 0, rank + rot), T)
         latent = ops.latent_attention(qa, H, rank, rot, batch.tok_req, batch.positions, pages.block_table,
-                                      site.cache, pages.page_size, self.scale, self.window or 0)
+                                      site.cache, pages.page_size, self.scale, self.window or 0,
+                                      plan=batch.plans.get(ops.LATENT_PLAN), max_ctx=batch.max_ctx)
         heads = torch.empty((T, H * vdim), dtype=self.dtype, device=qdg.device)
         gate = ops.Strided(qdg, q_cols + rank + rot, vdim) if self.gate else None
         ops.grouped_gemm(ops.Strided(latent, 0, rank), self.uv, ops.Strided(heads, 0, vdim), T, gate=gate)

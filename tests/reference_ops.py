@@ -208,7 +208,8 @@ def latent_prepare(proj, heads, dim, rot, rank, norm_weight, eps, positions, rop
                 cache[s // page, s % page] = row[t]
 
 
-def latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page_size, scale, window=0):
+def latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page_size, scale, window=0,
+                     plan=None, max_ctx=0):
     T = qa.shape[0]
     q = qa.view(T, heads, rank + rot).to(F64)
     out = torch.zeros(T, heads, rank, dtype=F64, device=qa.device)

@@ -365,3 +365,59 @@ def test_float32_logits_do_not_depend_on_the_cut():
     for other in runs[1:]:
         for key, row in runs[0].items():
             assert torch.equal(row, other[key]), f"{key}: the bits differ between two cuts"
+
+
+# ------------------------------------------------------------------ the matrix-core latent attention kernel
+@pytest.mark.parametrize("heads,rank,rot,page,window", [(4, 32, 16, 16, 0), (3, 48, 8, 4, 37), (16, 64, 32, 16, 100),
+                                                        (70, 16, 0, 8, 0), (9, 512, 64, 16, 130), (2, 208, 24, 32, 64)])
+def test_latent_attention_on_the_matrix_cores(heads, rank, rot, page, window):
+    """A step of portions (of 40, 2 and 17 tokens after histories of 150, 0 and 33) beside lone tokens
+    (after 299 and 64), against the plain version and against the general kernel; then the same
+    with the keys of every tile shared out over several workgroups."""
+    from lucciola_amd.engine.batch import HostLayout, Plan
+    g = torch.Generator().manual_seed(heads + rank)
+    history, fresh = [150, 0, 299, 33, 64], [40, 2, 1, 17, 1]
+    n_pages = sum(-(-(h + f) // page) for h, f in zip(history, fresh)) + 2
+    order = torch.randperm(n_pages, generator=g).tolist()
+    width = max(-(-(h + f) // page) for h, f in zip(history, fresh))
+    block_table = torch.full((len(history), width), -1, dtype=torch.int32)
+    cache = (torch.randn(n_pages, page, rank + rot, generator=g) * 0.5).bfloat16()
+    for r, (h, f) in enumerate(zip(history, fresh)):
+        for b in range(-(-(h + f) // page)):
+            block_table[r, b] = order.pop()
+    q_start = [0]
+    for f in fresh:
+        q_start.append(q_start[-1] + f)
+    T = q_start[-1]
+    tok_req = torch.tensor([r for r, f in enumerate(fresh) for _ in range(f)], dtype=torch.int32)
+    positions = torch.tensor([history[r] + i for r, f in enumerate(fresh) for i in range(f)], dtype=torch.int32)
+    qa = torch.randn(T, heads * (rank + rot), generator=g).bfloat16()
+    arrays, info = ops.plan_latent_attention(HostLayout(len(fresh), T, q_start, history, page, False))
+    plan = Plan({k: torch.from_numpy(v).to(DEV) for k, v in arrays.items()}, info)
+    want = reference_ops.latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page, 0.2, window)
+    args = (qa.to(DEV), heads, rank, rot, tok_req.to(DEV), positions.to(DEV), block_table.to(DEV), cache.to(DEV), page,
+            0.2, window)
+    plain = ops.latent_attention(*args)
+    close(plain.cpu(), want, torch.bfloat16, "general kernel")
+    assert ops.library().lc_latent_bf16_supported(rank, rot)
+    fast = ops.latent_attention(*args, plan=plan, max_ctx=300)
+    close(fast.cpu(), want, torch.bfloat16, "matrix-core kernel")
+    shared = ops.latent_attention(*args, plan=plan, max_ctx=1 << 20)       # a wide table: many shares, most of them empty
+    close(shared.cpu(), want, torch.bfloat16, "matrix-core kernel with shares")
+
+
+def test_matrix_core_path_is_the_one_that_serves():
+    """A bfloat16 engine with sizes the kernel takes runs it (and the general kernel when switched off),
+    with the same logits within rounding."""
+    cfg, page, weights, prompts, refs = case("C")
+    steps = traces.mixed(prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    fast = replay(make_runner(cfg, weights, page, blocks, "bfloat16", DEV), steps)
+    before = ops.latent_matrix_cores(False)
+    try:
+        slow = replay(make_runner(cfg, weights, page, blocks, "bfloat16", DEV), steps)
+    finally:
+        ops.latent_matrix_cores(before)
+    compare(fast, cfg, weights, prompts, TOL["bfloat16"], refs)
+    compare(slow, cfg, weights, prompts, TOL["bfloat16"], refs)
+    assert any(not torch.equal(fast[k], slow[k]) for k in fast), "both runs took the same kernel"
