@@ -24,6 +24,8 @@ namespace lc {
 constexpr int GG_N = 64, GG_K = 16, GG_CHUNK = 256, GG_PAD = 16;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+static thread_local int g_grouped_fast = 1;
+
 struct GroupedArgs {
     const void* x; long long ldx, x_group;
     const void* w;
@@ -187,6 +189,122 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_kernel(GroupedArgs a) {
             }
 }
 
+
+// The same products for bfloat16 operands on v_mfma_f32_16x16x32_bf16 (float32 sums over all of K
+// in order): steps of 32 k, both tiles in LDS as rows of 32 k (padded to 40: every operand is one
+// conflict-free 16-byte read), the next step's pieces in registers while this one is multiplied.
+// Rows and groups as above; K, the rows' strides and the groups' offsets must be multiples of 8.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int GH_K = 32, GH_STRIDE = GH_K + 8;
+
+template <typename TO, int BM, int WM, int WN>
+__global__ __launch_bounds__(256, 2) void gemm_grouped_bf16_kernel(GroupedArgs a) {
+    static_assert(WM * WN == 4, "four waves");
+    constexpr int BN = GG_N;
+    constexpr int TM = BM / 16 / WM, TN = BN / 16 / WN;
+    __shared__ __align__(16) bf16 xs[2][BM][GH_STRIDE];
+    __shared__ __align__(16) bf16 ws[2][BN][GH_STRIDE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
+    const int N = a.N, K = a.K;
+    int grp, r0, r_end;
+    if (a.row_start) {
+        const int tile = blockIdx.y;
+        if (tile >= a.tile_start[a.G]) return;
+        int lo = 0, hi = a.G - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (a.tile_start[mid] <= tile) lo = mid; else hi = mid - 1;
+        }
+        grp = lo;
+        r0 = a.row_start[grp] + (tile - a.tile_start[grp]) * BM;
+        r_end = a.row_start[grp + 1];
+    } else {
+        grp = blockIdx.z;
+        r0 = blockIdx.y * BM;
+        r_end = a.M;
+    }
+    const int n0 = blockIdx.x * BN;
+    const bf16* x = reinterpret_cast<const bf16*>(a.x) + (size_t)grp * a.x_group;
+    const bf16* w = reinterpret_cast<const bf16*>(a.w) + (size_t)grp * N * K;
+    const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
+    // loader: a thread brings one 16-byte piece (8 k) of a row of w and, where it has one, of x
+    const int lrow = tid >> 2, lk = (tid & 3) * 8;
+    const bool xlive = lrow < BM && r0 + lrow < r_end;
+    const bool wlive = n0 + lrow < N;
+    const int m_src = xlive ? r0 + lrow : r0;
+    const bf16* xrow = x + (size_t)(a.gather ? a.gather[m_src] : m_src) * a.ldx + lk;
+    const bf16* wrow = w + (size_t)(wlive ? n0 + lrow : 0) * K + lk;
+    bf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = static_cast<bf16>(0.f);
+    bf16x8 xr = zero, wr = zero;
+    auto fetch = [&](int k0) {
+        const bool in = k0 + lk < K;                // K % 8 == 0: a piece is whole or absent
+        xr = (xlive && in) ? *reinterpret_cast<const bf16x8*>(xrow + k0) : zero;
+        wr = (wlive && in) ? *reinterpret_cast<const bf16x8*>(wrow + k0) : zero;
+    };
+    auto put = [&](int stage) {
+        if (lrow < BM) *reinterpret_cast<bf16x8*>(&xs[stage][lrow][lk]) = xr;
+        *reinterpret_cast<bf16x8*>(&ws[stage][lrow][lk]) = wr;
+    };
+    floatx4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    int stage = 0;
+    fetch(0);
+    put(0);
+    for (int k0 = 0; k0 < K; k0 += GH_K) {
+        __syncthreads();
+        const bool more = k0 + GH_K < K;
+        if (more) fetch(k0 + GH_K);
+        bf16x8 av[TM], bv[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[i] = *reinterpret_cast<const bf16x8*>(&xs[stage][wm + 16 * i + col][8 * g]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = *reinterpret_cast<const bf16x8*>(&ws[stage][wn + 16 * j + col][8 * g]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        stage ^= 1;
+        if (more) put(stage);
+    }
+    // C = x . w^T with x as the first operand: the lane holds the rows 4 g + r, column col of a tile
+    TO* out = reinterpret_cast<TO*>(a.out) + (size_t)grp * a.out_group;
+    const bf16* gate = a.gate ? reinterpret_cast<const bf16*>(a.gate) + (size_t)grp * a.gate_group : nullptr;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = r0 + wm + 16 * i + 4 * g + r, n = n0 + wn + 16 * j + col;
+                if (m < r_end && n < N) {
+                    float v = acc[i][j][r];
+                    if (a.epilogue == ACT_SIGMOID_GATE) v *= sigmoid(to_f32(gate[(size_t)m * a.ldg + n]));
+                    else v = activate(v, a.epilogue);
+                    out[(size_t)m * a.ldo + n] = from_f32<TO>(v);
+                }
+            }
+}
+
+template <typename TO>
+static int launch_grouped_bf16(const GroupedArgs& a, int max_tiles, int small, hipStream_t stream) {
+    const int nb = (a.N + GG_N - 1) / GG_N;
+    if (small) {
+        dim3 grid(nb, a.row_start ? max_tiles : (a.M + 15) / 16, a.row_start ? 1 : a.G);
+        gemm_grouped_bf16_kernel<TO, 16, 1, 4><<<grid, 256, 0, stream>>>(a);
+    } else {
+        dim3 grid(nb, a.row_start ? max_tiles : (a.M + 63) / 64, a.row_start ? 1 : a.G);
+        gemm_grouped_bf16_kernel<TO, 64, 2, 2><<<grid, 256, 0, stream>>>(a);
+    }
+    LC_LAUNCH_CHECK("gemm_grouped_bf16");
+    return 0;
+}
+
 template <typename TX, typename TW, typename TO>
 static int launch_grouped(const GroupedArgs& a, int max_tiles, int small, hipStream_t stream) {
     const int nb = (a.N + GG_N - 1) / GG_N;
@@ -204,6 +322,14 @@ static int launch_grouped(const GroupedArgs& a, int max_tiles, int small, hipStr
 }  // namespace lc
 
 using namespace lc;
+
+// Tests and tuning: whether bfloat16 operands may take the bfloat16 matrix instruction (1, the default)
+// or always the true 32-bit product (0), for the calling thread.  Returns the setting before.
+LC_API int lc_gemm_grouped_fast(int on) {
+    const int before = g_grouped_fast;
+    if (on >= 0) g_grouped_fast = on ? 1 : 0;
+    return before;
+}
 
 // Rows of a tile: 16 where `small`, else 64; the lists' tile_start must have been made for it.
 LC_API int lc_gemm_grouped_tile_rows(int small) { return small ? 16 : 64; }
@@ -226,6 +352,12 @@ LC_API int lc_gemm_grouped(const void* x, int x_dt, long long ldx, long long x_g
     LC_CHECK(G <= 65535 && (row_start ? max_tiles : (M + 15) / 16) <= 65535, "grouped product: too many tiles");
     GroupedArgs a{x, ldx, x_group, w, out, ldo, out_group, M, N, K, G, gather, row_start, tile_start,
                   epilogue, gate, ldg, gate_group};
+    // bfloat16 operands whose pieces of 8 are whole and aligned: the bfloat16 matrix instruction
+    if (x_dt == DT_BF16 && w_dt == DT_BF16 && K % 8 == 0 && ldx % 8 == 0 && x_group % 8 == 0 &&
+        (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && g_grouped_fast) {
+        if (out_dt == DT_BF16) return launch_grouped_bf16<bf16>(a, max_tiles, small, stream);
+        if (out_dt == DT_F32) return launch_grouped_bf16<float>(a, max_tiles, small, stream);
+    }
     const int key = x_dt * 4 + w_dt * 2 + out_dt;
     switch (key) {
         case 0: return launch_grouped<float, float, float>(a, max_tiles, small, stream);

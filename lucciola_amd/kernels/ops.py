@@ -74,6 +74,7 @@ _SIGNATURES = {
     "lc_stream_add": "ppipiip",
     "lc_activation": "piiqp",
     "lc_gemm_grouped": "piqqpipiqqiiiipppiiipqqp",
+    "lc_gemm_grouped_fast": "i",
     "lc_latent_prepare": "piqiiiiipfppiipppp",
     "lc_latent_attention": "piiiiippppiifipp",
     "lc_latent_bf16_supported": "ii",
@@ -977,6 +978,12 @@ def grouped_gemm(x: Strided, w: torch.Tensor, out: Strided, rows: int, gate: Opt
           out.pointer(), _dt(out.tensor), out.tensor.shape[1], out.group, rows, N, K, G, None, None, None, 0,
           1 if rows <= 16 else 0, epilogue, gate.pointer() if gate is not None else None,
           gate.tensor.shape[1] if gate is not None else 0, gate.group if gate is not None else 0, _stream())
+
+
+def grouped_gemm_matrix_cores(on: bool) -> bool:
+    """Whether grouped products of bfloat16 operands may take the bfloat16 matrix instruction (the
+    default) or always run as true 32-bit products; for tests and tuning.  Returns the setting before."""
+    return bool(library().lc_gemm_grouped_fast(1 if on else 0))
 
 
 # ------------------------------------------------------------------------------ latent attention

@@ -67,11 +67,14 @@ def test_stream_add_and_activations():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,G,N,K", [(1, 3, 21, 7), (16, 2, 64, 32), (77, 5, 18, 300), (130, 1, 100, 9)])
-def test_grouped_product_over_heads(dtype, rows, G, N, K):
+@pytest.mark.parametrize("rows,G,N,K,pad_x,gap", [(1, 3, 21, 7, 5, 2), (16, 2, 64, 32, 5, 2), (77, 5, 18, 300, 5, 2),
+                                                  (130, 1, 100, 9, 5, 2),
+                                                  # whole 16-byte pieces: in bfloat16 the bfloat16 matrix instruction
+                                                  (3, 4, 96, 32, 8, 8), (70, 3, 40, 136, 16, 0), (200, 2, 130, 512, 0, 64)])
+def test_grouped_product_over_heads(dtype, rows, G, N, K, pad_x, gap):
     g = torch.Generator().manual_seed(rows * 7 + G)
-    pad_x, pad_o = 5, 3
-    x = torch.randn(rows, pad_x + G * (K + 2), generator=g).to(dtype)
+    pad_o = 3
+    x = torch.randn(rows, pad_x + G * (K + gap), generator=g).to(dtype)
     w = torch.randn(G, N, K, generator=g).bfloat16()
     gate = torch.randn(rows, G * N + 4, generator=g).to(dtype)
     for use_gate, act in ((False, None), (True, None), (False, "relu_squared")):
@@ -79,8 +82,8 @@ def test_grouped_product_over_heads(dtype, rows, G, N, K):
         out_dev = torch.zeros(rows, pad_o + G * N, dtype=dtype, device=DEV)
         gate_ref = ops.Strided(gate, 4, N) if use_gate else None
         gate_dev = ops.Strided(gate.to(DEV), 4, N) if use_gate else None
-        reference_ops.grouped_gemm(ops.Strided(x, pad_x, K + 2), w, ops.Strided(out_ref, pad_o, N), rows, gate_ref, act)
-        ops.grouped_gemm(ops.Strided(x.to(DEV), pad_x, K + 2), w.to(DEV), ops.Strided(out_dev, pad_o, N), rows, gate_dev, act)
+        reference_ops.grouped_gemm(ops.Strided(x, pad_x, K + gap), w, ops.Strided(out_ref, pad_o, N), rows, gate_ref, act)
+        ops.grouped_gemm(ops.Strided(x.to(DEV), pad_x, K + gap), w.to(DEV), ops.Strided(out_dev, pad_o, N), rows, gate_dev, act)
         close(out_dev.cpu(), out_ref, dtype, f"grouped product gate={use_gate} act={act}")
         assert float(out_dev[:, :pad_o].abs().max()) == 0.0, "columns before the first group were written"
 
