@@ -1,5 +1,5 @@
 // Latent attention in bfloat16 on the matrix cores (v_mfma_f32_16x16x32_bf16), for latents of a
-// multiple of 16 entries (up to 512) and rows [c | k_r] of a multiple of 8 (up to 640).
+// multiple of 16 entries (up to 512) and rows [c | k_r] of a multiple of 8 (up to 576).
 //
 // As in latent.hip every head of a token attends over the same cached rows, with the query in the
 // latent's space; scores, maxima, exponentials and sums are float32, the weights are rounded to
@@ -44,6 +44,7 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     const int kstride = Dp + LM_KPAD;                       // bf16 a staged row
     bf16* ks_lds = reinterpret_cast<bf16*>(lds_raw);        // [LM_STAGE][kstride]
     bf16* vt_lds = ks_lds + LM_STAGE * kstride;             // [R][LM_VSTRIDE]
+    int* rows_lds = reinterpret_cast<int*>(vt_lds + (size_t)R * LM_VSTRIDE);    // [2][LM_STAGE]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
     const int* tile = tiles + 4 * blockIdx.x;
     const int t0 = tile[0], ntok = tile[1], req = tile[2], p0 = tile[3];
@@ -86,28 +87,43 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     float m_run = -INFINITY, l_run = 0.f;
 
     const int pieces = Dk / 8;                              // 16-byte pieces of a row
+    // where the keys of a stage lie (page * page size + offset), looked up a stage ahead: a key
+    // behind the tile's last is that last key once more (finite, and no query sees it)
+    auto row_of = [&](int j) {
+        j = min(j, p_last);
+        return table[j / page_size] * page_size + j % page_size;
+    };
+    if (tid < LM_STAGE && s_begin < s_end) rows_lds[tid] = row_of(j_lo + s_begin * LM_STAGE + tid);
+    constexpr int PER = (LM_STAGE * KS * 4 + LM_THREADS - 1) / LM_THREADS;     // pieces of the rows a thread brings
     for (int s = s_begin; s < s_end; ++s) {
         const int c0 = j_lo + s * LM_STAGE;
-        __syncthreads();                                    // the stage before has been read
-        // rows: piece by piece (a key behind the tile's last is that last key once more: finite, unread)
-        for (int i = tid; i < LM_STAGE * pieces; i += LM_THREADS) {
+        const int* rows = rows_lds + ((s - s_begin) & 1) * LM_STAGE;
+        __syncthreads();                                    // the stage before has been read; rows are there
+        // rows, piece by piece: all of a thread's loads are on their way before the first is stored
+        bf16x8 got[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid + u * LM_THREADS;
             const int key = i / pieces, piece = i - key * pieces;
-            const int j = min(c0 + key, p_last);
-            const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-            *reinterpret_cast<bf16x8*>(ks_lds + key * kstride + piece * 8) =
-                *reinterpret_cast<const bf16x8*>(cache + row * Dk + piece * 8);
+            if (key < LM_STAGE) got[u] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[key] * Dk + piece * 8);
         }
-        // latent entries, transposed: a thread takes eight entries of the eight keys of a lane
-        // group's run and writes, for each entry, the run as one piece
+        if (tid < LM_STAGE && s + 1 < s_end)                // the next stage's rows: asked for now, needed a stage on
+            rows_lds[((s + 1 - s_begin) & 1) * LM_STAGE + tid] = row_of(c0 + LM_STAGE + tid);
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid + u * LM_THREADS;
+            const int key = i / pieces, piece = i - key * pieces;
+            if (key < LM_STAGE) *reinterpret_cast<bf16x8*>(ks_lds + key * kstride + piece * 8) = got[u];
+        }
+        __syncthreads();
+        // latent entries, transposed, from the rows just staged: a thread takes eight entries of the
+        // eight keys of a lane group's run and writes, for each entry, the run as one piece
         for (int i = tid; i < (R / 8) * 4; i += LM_THREADS) {
             const int gg = i & 3, dp = i >> 2;
             bf16x8 in[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int j = min(c0 + stage_key(gg, k), p_last);
-                const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-                in[k] = *reinterpret_cast<const bf16x8*>(cache + row * Dk + dp * 8);
-            }
+            for (int k = 0; k < 8; ++k)
+                in[k] = *reinterpret_cast<const bf16x8*>(ks_lds + stage_key(gg, k) * kstride + dp * 8);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 bf16x8 run;
@@ -200,29 +216,32 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
 // One workgroup per (token, head): the shares' sums, taken in from the first.
 __global__ void latent_attention_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                              int splits, int R, bf16* __restrict__ out) {
+    __shared__ float weight[64];
+    __shared__ float total;
     const size_t qi = blockIdx.x;
-    float M = -INFINITY;
-    for (int z = 0; z < splits; ++z) M = fmaxf(M, part_ml[(qi * splits + z) * 2]);
-    float L = 0.f;
-    for (int z = 0; z < splits; ++z) {
-        const float m = part_ml[(qi * splits + z) * 2];
-        if (m != -INFINITY) L = fmaf(part_ml[(qi * splits + z) * 2 + 1], expf(m - M), L);
+    if (threadIdx.x < 64) {
+        const int z = threadIdx.x;
+        const float m = z < splits ? part_ml[(qi * splits + z) * 2] : -INFINITY;
+        const float M = wave_max(m);
+        const float w = m == -INFINITY ? 0.f : expf(m - M);
+        weight[z] = w;
+        const float L = wave_sum(z < splits ? part_ml[(qi * splits + z) * 2 + 1] * w : 0.f);
+        if (z == 0) total = L;
     }
+    __syncthreads();
+    const float inv = 1.f / total;
     for (int d = threadIdx.x; d < R; d += blockDim.x) {
         float acc = 0.f;
-        for (int z = 0; z < splits; ++z) {
-            const float m = part_ml[(qi * splits + z) * 2];
-            if (m != -INFINITY) acc = fmaf(part_o[(qi * splits + z) * R + d], expf(m - M), acc);
-        }
-        out[qi * R + d] = static_cast<bf16>(acc / L);
+        for (int z = 0; z < splits; ++z) acc = fmaf(part_o[(qi * splits + z) * R + d], weight[z], acc);
+        out[qi * R + d] = static_cast<bf16>(acc * inv);
     }
 }
 
 static bool shape_of(int R, int rot, int* nr, int* ks) {
     const int Dk = R + rot;
-    if (R <= 0 || R % 16 || Dk % 8 || R > 512 || Dk > 640) return false;
+    if (R <= 0 || R % 16 || Dk % 8 || R > 512 || Dk > 576) return false;
     const int need_nr = R / 16, need_ks = (Dk + 31) / 32;
-    const int classes[4][2] = {{4, 4}, {8, 8}, {16, 12}, {32, 20}};
+    const int classes[4][2] = {{4, 4}, {8, 8}, {16, 12}, {32, 18}};
     for (auto& c : classes)
         if (need_nr <= c[0] && need_ks <= c[1]) { *nr = c[0]; *ks = c[1]; return true; }
     return false;
@@ -267,7 +286,8 @@ LC_API int lc_latent_attention_bf16(const void* qa, int T, int H, int R, int rot
     const int blocks_y = any_portion ? (H + 3) / 4 : (H + 63) / 64;
     LC_CHECK(blocks_y <= 65535, "latent attention: too many heads (%d)", H);
     const dim3 grid(num_tiles, blocks_y, splits);
-    const size_t lds = sizeof(bf16) * ((size_t)LM_STAGE * (ks * 32 + LM_KPAD) + (size_t)R * LM_VSTRIDE);
+    const size_t lds = sizeof(bf16) * ((size_t)LM_STAGE * (ks * 32 + LM_KPAD) + (size_t)R * LM_VSTRIDE) +
+                       sizeof(int) * 2 * LM_STAGE;
 #define LC_LM_LAUNCH(NR, KS)                                                                                       \
     do {                                                                                                           \
         if (lds > 64 * 1024)                                                                                       \
@@ -281,11 +301,11 @@ LC_API int lc_latent_attention_bf16(const void* qa, int T, int H, int R, int rot
     if (nr == 4) LC_LM_LAUNCH(4, 4);
     else if (nr == 8) LC_LM_LAUNCH(8, 8);
     else if (nr == 16) LC_LM_LAUNCH(16, 12);
-    else LC_LM_LAUNCH(32, 20);
+    else LC_LM_LAUNCH(32, 18);
 #undef LC_LM_LAUNCH
     LC_LAUNCH_CHECK("latent_attention_bf16");
     if (splits > 1) {
-        latent_attention_join_kernel<<<T * H, 128, 0, stream>>>(part_o, part_ml, splits, R, (bf16*)out);
+        latent_attention_join_kernel<<<T * H, 256, 0, stream>>>(part_o, part_ml, splits, R, (bf16*)out);
         LC_LAUNCH_CHECK("latent_attention_join");
     }
     return 0;

@@ -64,7 +64,9 @@ LC_API int lc_dynamic_tanh(float* h, const void* delta, const int* rows, const f
     if (R == 0) return 0;
     LC_CHECK(h && w && b && out, "dynamic_tanh: null pointer");
     LC_CHECK(!(rows && write_h), "dynamic_tanh: gathered rows cannot be written back");
-    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    // a row's entries are independent: with few rows, as many threads a row as it has pairs of
+    // entries, so that no thread walks the row load after load
+    const int threads = (R <= 256 && n >= 2048) ? 1024 : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
     if (dt == DT_F32)
         dynamic_tanh_kernel<float><<<R, threads, 0, stream>>>(h, (const float*)delta, rows, w, b, alpha, (float*)out, n, write_h);
     else if (dt == DT_BF16)

@@ -1100,7 +1100,7 @@ def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req:
     if qa.dtype == torch.bfloat16 and plan is not None and _latent_fast.on and rank * heads >= 1024:
         _say_once(("latent attention", rank, rot),
                   f"bfloat16 latent attention with a latent of {rank} and {rot} rotated entries has no matrix-core "
-                  "kernel (a latent of a multiple of 16 up to 512, rows of a multiple of 8 up to 640): the general "
+                  "kernel (a latent of a multiple of 16 up to 512, rows of a multiple of 8 up to 576): the general "
                   "kernel runs, correct and many times slower")
     _call("lc_latent_attention", _ptr(qa), _dt(qa), T, heads, rank, rot, _ptr(cache), _ptr(tok_req),
           _ptr(positions), _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
