@@ -1,14 +1,15 @@
 // Latent attention in bfloat16 on the matrix cores (v_mfma_f32_16x16x32_bf16), for latents of a
-// multiple of 16 entries (up to 512) and rows [c | k_r] of a multiple of 8 (up to 576).
+// multiple of 16 entries (up to 512) and rows [c | k_r] of a multiple of 8 (up to 576, of which up
+// to 128 rotated).
 //
 // As in latent.hip every head of a token attends over the same cached rows, with the query in the
 // latent's space; scores, maxima, exponentials and sums are float32, the weights are rounded to
 // bfloat16 for the product with the rows (as the other matrix-core attention kernels do).
 //
 // A work item is a tile of the planner's list: up to 16 tokens in a row of one request (a piece
-// of a prompt's portion), or one token (a decoding request).  A workgroup of four waves serves a
-// tile and some heads: a wave has 16 query columns, which are the tile's tokens for one head (wave
-// w: head h0 + w) or, for a lone token, 16 heads (wave w: heads h0 + 16 w ...).  All waves read
+// of a prompt's portion), or one token (a decoding request).  A workgroup of four pairs of waves serves a
+// tile and some heads: a pair has 16 query columns, which are the tile's tokens for one head (pair
+// w: head h0 + w) or, for a lone token, 16 heads (pair w: heads h0 + 16 w ...).  All waves read
 // the same keys: a stage of 32 cached rows is brought into LDS once, as rows (the operand of
 // S^T = K . Q^T) and, its latent part, transposed ([entry][key], the operand of O^T = C^T . P^T),
 // so that every operand is one 16-byte LDS read.  S^T leaves a lane with the keys 4 g + r of a
@@ -24,8 +25,10 @@ namespace lc {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int LM_THREADS = 256;
+constexpr int LM_THREADS = 512;       // eight waves: four pairs, a pair shares its query columns
+constexpr int LM_STAGERS = 256;       // threads that bring the latent part of a stage
 constexpr int LM_STAGE = 32;          // keys of a stage
+constexpr int LM_ROT_MOST = 128;      // rotated entries of a row, at most
 constexpr int LM_KPAD = 8;            // bf16 of padding behind a staged row
 constexpr int LM_VSTRIDE = LM_STAGE + 8;   // bf16 between two entries' key runs in the transposed stage
 
@@ -45,7 +48,12 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     bf16* ks_lds = reinterpret_cast<bf16*>(lds_raw);        // [LM_STAGE][kstride]
     bf16* vt_lds = ks_lds + LM_STAGE * kstride;             // [R][LM_VSTRIDE]
     int* rows_lds = reinterpret_cast<int*>(vt_lds + (size_t)R * LM_VSTRIDE);    // [2][LM_STAGE]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
+    // a pair of waves has the same 16 query columns: both make the scores and weights (what one
+    // would have to hand to the other costs more than making them twice), each sums one half of the
+    // latent's entries, so that a wave's sums and queries fit half of a SIMD's registers and two
+    // waves share every SIMD
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 7, half = (tid >> 6) & 1, col = lane & 15, g = lane >> 4;
+    constexpr int NH = NR / 2;
     const int* tile = tiles + 4 * blockIdx.x;
     const int t0 = tile[0], ntok = tile[1], req = tile[2], p0 = tile[3];
     const bool lone = ntok == 1;
@@ -56,6 +64,10 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     const bool q_live = q_tok < ntok && q_head < H;
     const bool wave_live = lone ? h0 + 16 * wave < H : h0 + wave < H;
     const int p_q = p0 + q_tok;
+    // the keys the lane's column sees: q_lo .. q_hi (none for a column that is not there)
+    const int q_hi = q_live ? p_q : -1;
+    const int q_lo = window > 0 ? p_q - window + 1 : 0;
+    const float scale_log2 = scale * 1.4426950408889634f;
     const int p_last = p0 + ntok - 1;
     const int j_lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
     const int stages = (p_last - j_lo) / LM_STAGE + 1;
@@ -81,49 +93,57 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
         const int key = i / (Dp - Dk), e = Dk + i % (Dp - Dk);
         ks_lds[key * kstride + e] = static_cast<bf16>(0.f);
     }
-    floatx4 o[NR];
+    floatx4 o[NH];                                          // entries 16 (half NH + d) ... of the latent
 #pragma unroll
-    for (int d = 0; d < NR; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int d = 0; d < NH; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int pieces = Dk / 8;                              // 16-byte pieces of a row
     // where the keys of a stage lie (page * page size + offset), looked up a stage ahead: a key
     // behind the tile's last is that last key once more (finite, and no query sees it)
     auto row_of = [&](int j) {
         j = min(j, p_last);
         return table[j / page_size] * page_size + j % page_size;
     };
-    if (tid < LM_STAGE && s_begin < s_end) rows_lds[tid] = row_of(j_lo + s_begin * LM_STAGE + tid);
-    constexpr int PER = (LM_STAGE * KS * 4 + LM_THREADS - 1) / LM_THREADS;     // pieces of the rows a thread brings
-    for (int s = s_begin; s < s_end; ++s) {
-        const int c0 = j_lo + s * LM_STAGE;
-        const int* rows = rows_lds + ((s - s_begin) & 1) * LM_STAGE;
-        __syncthreads();                                    // the stage before has been read; rows are there
-        // rows, piece by piece: all of a thread's loads are on their way before the first is stored
-        bf16x8 got[PER];
+    // Staging.  A thread brings, of the latent part, eight entries of the eight keys of one lane
+    // group's run (R / 8 x 4 such pieces of work, at most one a thread) and stores them twice: as they
+    // are into the rows, and transposed (for each entry the run of eight keys as one piece).  Of the
+    // rotated part behind the latent it brings single 16-byte pieces.  All of it is asked for a stage
+    // ahead and travels while the stage before is multiplied.
+    const int gg = tid & 3, dp = tid >> 2;
+    const bool has_c = tid < LM_STAGERS && dp * 8 < R;
+    const int rot_pieces = rot / 8;                         // 16-byte pieces of a row's rotated part
+    constexpr int RP = LM_STAGE * (LM_ROT_MOST / 8) / (LM_THREADS - LM_STAGERS);   // such pieces a thread, at most
+    bf16x8 in[8], extra[RP];
+    int ex_key[RP], ex_piece[RP];
 #pragma unroll
-        for (int u = 0; u < PER; ++u) {
-            const int i = tid + u * LM_THREADS;
-            const int key = i / pieces, piece = i - key * pieces;
-            if (key < LM_STAGE) got[u] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[key] * Dk + piece * 8);
-        }
-        if (tid < LM_STAGE && s + 1 < s_end)                // the next stage's rows: asked for now, needed a stage on
-            rows_lds[((s + 1 - s_begin) & 1) * LM_STAGE + tid] = row_of(c0 + LM_STAGE + tid);
-#pragma unroll
-        for (int u = 0; u < PER; ++u) {
-            const int i = tid + u * LM_THREADS;
-            const int key = i / pieces, piece = i - key * pieces;
-            if (key < LM_STAGE) *reinterpret_cast<bf16x8*>(ks_lds + key * kstride + piece * 8) = got[u];
-        }
-        __syncthreads();
-        // latent entries, transposed, from the rows just staged: a thread takes eight entries of the
-        // eight keys of a lane group's run and writes, for each entry, the run as one piece
-        for (int i = tid; i < (R / 8) * 4; i += LM_THREADS) {
-            const int gg = i & 3, dp = i >> 2;
-            bf16x8 in[8];
+    for (int u = 0; u < RP; ++u) {
+        const int i = tid - LM_STAGERS + u * (LM_THREADS - LM_STAGERS);      // the other threads bring these
+        ex_key[u] = (rot_pieces && tid >= LM_STAGERS) ? i / rot_pieces : LM_STAGE;
+        ex_piece[u] = rot_pieces ? i - ex_key[u] * rot_pieces : 0;
+    }
+    auto ask = [&](const int* rows) {
+        if (has_c)
 #pragma unroll
             for (int k = 0; k < 8; ++k)
-                in[k] = *reinterpret_cast<const bf16x8*>(ks_lds + stage_key(gg, k) * kstride + dp * 8);
+                in[k] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[stage_key(gg, k)] * Dk + dp * 8);
+#pragma unroll
+        for (int u = 0; u < RP; ++u)
+            if (ex_key[u] < LM_STAGE)
+                extra[u] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[ex_key[u]] * Dk + R + ex_piece[u] * 8);
+    };
+    if (s_begin < s_end) {
+        if (tid < LM_STAGE) rows_lds[tid] = row_of(j_lo + s_begin * LM_STAGE + tid);
+        __syncthreads();
+        ask(rows_lds);
+    }
+    for (int s = s_begin; s < s_end; ++s) {
+        const int c0 = j_lo + s * LM_STAGE;
+        int* rows_next = rows_lds + ((s + 1 - s_begin) & 1) * LM_STAGE;
+        __syncthreads();                                    // the stage before has been read
+        if (has_c) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                *reinterpret_cast<bf16x8*>(ks_lds + stage_key(gg, k) * kstride + dp * 8) = in[k];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 bf16x8 run;
@@ -132,7 +152,13 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
                 *reinterpret_cast<bf16x8*>(vt_lds + (dp * 8 + e) * LM_VSTRIDE + gg * 8) = run;
             }
         }
+#pragma unroll
+        for (int u = 0; u < RP; ++u)
+            if (ex_key[u] < LM_STAGE)
+                *reinterpret_cast<bf16x8*>(ks_lds + ex_key[u] * kstride + R + ex_piece[u] * 8) = extra[u];
+        if (tid < LM_STAGE && s + 1 < s_end) rows_next[tid] = row_of(c0 + LM_STAGE + tid);
         __syncthreads();
+        if (s + 1 < s_end) ask(rows_next);                  // the next stage's rows travel while this one is multiplied
         if (!wave_live) continue;
         // S^T = K . Q^T: two tiles of 16 keys
         floatx4 sc[2];
@@ -145,29 +171,29 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
                 sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + x * 32), qf[x],
                                                                 sc[kt], 0, 0, 0);
         }
-        // the lane holds the keys c0 + 16 kt + 4 g + r of its column
+        // the lane holds the keys c0 + 16 kt + 4 g + r of its column; scores in units of log 2, so that
+        // every exponential is one instruction
         float mx = -INFINITY;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = c0 + 16 * kt + 4 * g + r;
-                const bool seen = q_live && j <= p_q && (window <= 0 || j > p_q - window);
-                sc[kt][r] = seen ? sc[kt][r] * scale : -INFINITY;
+                sc[kt][r] = (j >= q_lo && j <= q_hi) ? sc[kt][r] * scale_log2 : -INFINITY;
                 mx = fmaxf(mx, sc[kt][r]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
         mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = expf(m_run - m_safe);           // 0 while the column has seen no key (its sums are 0)
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);   // 0 while the column has seen no key (its sums are 0)
         float sum = 0.f;
         bf16x8 pb;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float pj = expf(sc[kt][r] - m_safe);
+                const float pj = __builtin_amdgcn_exp2f(sc[kt][r] - m_safe);
                 sum += pj;
                 pb[4 * kt + r] = static_cast<bf16>(pj);
             }
@@ -178,12 +204,12 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         // O^T += C^T . P^T
 #pragma unroll
-        for (int d = 0; d < NR; ++d)
-            if (d * 16 < R) {
+        for (int d = 0; d < NH; ++d)
+            if ((half * NH + d) * 16 < R) {
                 if (rescale)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) o[d][r] *= alpha;
-                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt_lds + (d * 16 + col) * LM_VSTRIDE + 8 * g);
+                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt_lds + ((half * NH + d) * 16 + col) * LM_VSTRIDE + 8 * g);
                 o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[d], 0, 0, 0);
             }
     }
@@ -193,20 +219,20 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     if (splits == 1) {
         const float inv = 1.f / l_run;
 #pragma unroll
-        for (int d = 0; d < NR; ++d)
-            if (d * 16 < R) {
-                bf16* dst = out + qi * R + d * 16 + 4 * g;
+        for (int d = 0; d < NH; ++d)
+            if ((half * NH + d) * 16 < R) {
+                bf16* dst = out + qi * R + (half * NH + d) * 16 + 4 * g;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) dst[r] = static_cast<bf16>(o[d][r] * inv);
             }
     } else {
         float* dst = part_o + (qi * splits + blockIdx.z) * R;
 #pragma unroll
-        for (int d = 0; d < NR; ++d)
-            if (d * 16 < R)
+        for (int d = 0; d < NH; ++d)
+            if ((half * NH + d) * 16 < R)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) dst[d * 16 + 4 * g + r] = o[d][r];
-        if (g == 0) {
+                for (int r = 0; r < 4; ++r) dst[(half * NH + d) * 16 + 4 * g + r] = o[d][r];
+        if (g == 0 && half == 0) {
             part_ml[(qi * splits + blockIdx.z) * 2] = m_run;
             part_ml[(qi * splits + blockIdx.z) * 2 + 1] = l_run;
         }
@@ -223,7 +249,7 @@ __global__ void latent_attention_join_kernel(const float* __restrict__ part_o, c
         const int z = threadIdx.x;
         const float m = z < splits ? part_ml[(qi * splits + z) * 2] : -INFINITY;
         const float M = wave_max(m);
-        const float w = m == -INFINITY ? 0.f : expf(m - M);
+        const float w = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);     // the maxima are in units of log 2
         weight[z] = w;
         const float L = wave_sum(z < splits ? part_ml[(qi * splits + z) * 2 + 1] * w : 0.f);
         if (z == 0) total = L;
@@ -239,7 +265,7 @@ __global__ void latent_attention_join_kernel(const float* __restrict__ part_o, c
 
 static bool shape_of(int R, int rot, int* nr, int* ks) {
     const int Dk = R + rot;
-    if (R <= 0 || R % 16 || Dk % 8 || R > 512 || Dk > 576) return false;
+    if (R <= 0 || R % 16 || Dk % 8 || R > 512 || Dk > 576 || rot > LM_ROT_MOST) return false;
     const int need_nr = R / 16, need_ks = (Dk + 31) / 32;
     const int classes[4][2] = {{4, 4}, {8, 8}, {16, 12}, {32, 18}};
     for (auto& c : classes)

@@ -1056,6 +1056,9 @@ def plan_latent_attention(layout):
         first, n = layout.q_start[r], layout.q_start[r + 1] - layout.q_start[r]
         for t0 in range(0, n, LATENT_TILE):
             tiles.append((first + t0, min(LATENT_TILE, n - t0), r, layout.first_position[r] + t0))
+    # the tiles that see the most keys first: the kernel's workgroups start in this order, and whoever
+    # is done takes the longest that is left (the order changes no tile's result)
+    tiles.sort(key=lambda t: -(t[3] + t[1]))
     return ({"tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)},
             {"any_portion": any(t[1] > 1 for t in tiles), "num_tiles": len(tiles)})
 
@@ -1100,7 +1103,7 @@ def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req:
     if qa.dtype == torch.bfloat16 and plan is not None and _latent_fast.on and rank * heads >= 1024:
         _say_once(("latent attention", rank, rot),
                   f"bfloat16 latent attention with a latent of {rank} and {rot} rotated entries has no matrix-core "
-                  "kernel (a latent of a multiple of 16 up to 512, rows of a multiple of 8 up to 576): the general "
+                  "kernel (a latent of a multiple of 16 up to 512, rows of a multiple of 8 up to 576, at most 128 rotated entries): the general "
                   "kernel runs, correct and many times slower")
     _call("lc_latent_attention", _ptr(qa), _dt(qa), T, heads, rank, rot, _ptr(cache), _ptr(tok_req),
           _ptr(positions), _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
