@@ -23,17 +23,17 @@
 namespace lc {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int LM_THREADS = 512;       // eight waves: four pairs, a pair shares its query columns
-constexpr int LM_STAGERS = 256;       // threads that bring the latent part of a stage
 constexpr int LM_STAGE = 32;          // keys of a stage
 constexpr int LM_ROT_MOST = 128;      // rotated entries of a row, at most
 constexpr int LM_KPAD = 8;            // bf16 of padding behind a staged row
 constexpr int LM_VSTRIDE = LM_STAGE + 8;   // bf16 between two entries' key runs in the transposed stage
 
-// the key, counted from the stage's first, that lies at place i of lane group g's run of eight
-__device__ __forceinline__ int stage_key(int g, int i) { return i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4); }
+// (of a stage's 32 keys, lane group g's run of eight in the transposed stage is the keys 4 g ... 4 g + 3
+// and 16 + 4 g ... 16 + 4 g + 3: the keys of its two score tiles, which its weights are made of)
 
 // NR: tiles of 16 latent entries a wave keeps sums for; KS: steps of 32 row entries of a score
 template <int NR, int KS>
@@ -98,41 +98,47 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     for (int d = 0; d < NH; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    // where the keys of a stage lie (page * page size + offset), looked up a stage ahead: a key
+    // where the keys of a stage lie (page * page size + offset): a key
     // behind the tile's last is that last key once more (finite, and no query sees it)
     auto row_of = [&](int j) {
         j = min(j, p_last);
         return table[j / page_size] * page_size + j % page_size;
     };
-    // Staging.  A thread brings, of the latent part, eight entries of the eight keys of one lane
-    // group's run (R / 8 x 4 such pieces of work, at most one a thread) and stores them twice: as they
-    // are into the rows, and transposed (for each entry the run of eight keys as one piece).  Of the
-    // rotated part behind the latent it brings single 16-byte pieces.  All of it is asked for a stage
-    // ahead and travels while the stage before is multiplied.
-    const int gg = tid & 3, dp = tid >> 2;
-    const bool has_c = tid < LM_STAGERS && dp * 8 < R;
+    // Staging.  A thread brings, of the latent part, eight entries of four keys: one half of a lane
+    // group's run of eight (R / 8 x 8 such pieces of work, at most one a thread), and stores them
+    // twice: as they are into the rows, and transposed (for each entry its half of the run as one
+    // 8-byte piece).  Of the rotated part behind the latent it brings single 16-byte pieces.  All of
+    // it is asked for a stage ahead and travels while the stage before is multiplied.
+    const int gg = tid & 3, hh = (tid >> 2) & 1, dp = tid >> 3;
+    const bool has_c = dp * 8 < R;
     const int rot_pieces = rot / 8;                         // 16-byte pieces of a row's rotated part
-    constexpr int RP = LM_STAGE * (LM_ROT_MOST / 8) / (LM_THREADS - LM_STAGERS);   // such pieces a thread, at most
-    bf16x8 in[8], extra[RP];
+    constexpr int RP = LM_STAGE * (LM_ROT_MOST / 8) / LM_THREADS;             // such pieces a thread, at most
+    bf16x8 in[4], extra[RP];
     int ex_key[RP], ex_piece[RP];
 #pragma unroll
     for (int u = 0; u < RP; ++u) {
-        const int i = tid - LM_STAGERS + u * (LM_THREADS - LM_STAGERS);      // the other threads bring these
-        ex_key[u] = (rot_pieces && tid >= LM_STAGERS) ? i / rot_pieces : LM_STAGE;
+        const int i = tid + u * LM_THREADS;
+        ex_key[u] = rot_pieces ? i / rot_pieces : LM_STAGE;
         ex_piece[u] = rot_pieces ? i - ex_key[u] * rot_pieces : 0;
     }
     auto ask = [&](const int* rows) {
         if (has_c)
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
-                in[k] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[stage_key(gg, k)] * Dk + dp * 8);
+            for (int k = 0; k < 4; ++k)
+                in[k] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[16 * hh + 4 * gg + k] * Dk + dp * 8);
 #pragma unroll
         for (int u = 0; u < RP; ++u)
             if (ex_key[u] < LM_STAGE)
                 extra[u] = *reinterpret_cast<const bf16x8*>(cache + (size_t)rows[ex_key[u]] * Dk + R + ex_piece[u] * 8);
     };
+    // the rows of stage s + 2 are looked up while stage s is staged, wait in a register and reach
+    // LDS at the top of stage s + 1, whose loads for stage s + 2 read them: no look-up is waited for
+    int row_ahead = 0;
     if (s_begin < s_end) {
-        if (tid < LM_STAGE) rows_lds[tid] = row_of(j_lo + s_begin * LM_STAGE + tid);
+        if (tid < LM_STAGE) {
+            rows_lds[tid] = row_of(j_lo + s_begin * LM_STAGE + tid);
+            if (s_begin + 1 < s_end) row_ahead = row_of(j_lo + (s_begin + 1) * LM_STAGE + tid);
+        }
         __syncthreads();
         ask(rows_lds);
     }
@@ -140,36 +146,55 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
         const int c0 = j_lo + s * LM_STAGE;
         int* rows_next = rows_lds + ((s + 1 - s_begin) & 1) * LM_STAGE;
         __syncthreads();                                    // the stage before has been read
+        if (tid < LM_STAGE && s + 1 < s_end) {
+            rows_next[tid] = row_ahead;
+            if (s + 2 < s_end) row_ahead = row_of(c0 + 2 * LM_STAGE + tid);
+        }
         if (has_c) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
-                *reinterpret_cast<bf16x8*>(ks_lds + stage_key(gg, k) * kstride + dp * 8) = in[k];
+            for (int k = 0; k < 4; ++k)
+                *reinterpret_cast<bf16x8*>(ks_lds + (16 * hh + 4 * gg + k) * kstride + dp * 8) = in[k];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                bf16x8 run;
+                bf16x4 run;
 #pragma unroll
-                for (int k = 0; k < 8; ++k) run[k] = in[k][e];
-                *reinterpret_cast<bf16x8*>(vt_lds + (dp * 8 + e) * LM_VSTRIDE + gg * 8) = run;
+                for (int k = 0; k < 4; ++k) run[k] = in[k][e];
+                *reinterpret_cast<bf16x4*>(vt_lds + (dp * 8 + e) * LM_VSTRIDE + gg * 8 + hh * 4) = run;
             }
         }
 #pragma unroll
         for (int u = 0; u < RP; ++u)
             if (ex_key[u] < LM_STAGE)
                 *reinterpret_cast<bf16x8*>(ks_lds + ex_key[u] * kstride + R + ex_piece[u] * 8) = extra[u];
-        if (tid < LM_STAGE && s + 1 < s_end) rows_next[tid] = row_of(c0 + LM_STAGE + tid);
         __syncthreads();
         if (s + 1 < s_end) ask(rows_next);                  // the next stage's rows travel while this one is multiplied
         if (!wave_live) continue;
-        // S^T = K . Q^T: two tiles of 16 keys
+        // S^T = K . Q^T: two tiles of 16 keys.  The operands of a batch of products are all asked of
+        // LDS before the first product (a wave that is alone on its SIMD would otherwise wait for
+        // every read in turn), and the two tiles' products alternate
         floatx4 sc[2];
+        sc[0] = sc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        {
+            const bf16* krow = ks_lds + col * kstride + 8 * g;
+            constexpr int QB = 3;                           // steps of 32 entries a batch, for both tiles
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            sc[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-            const bf16* krow = ks_lds + (kt * 16 + col) * kstride + 8 * g;
+            for (int x0 = 0; x0 < KS; x0 += QB) {
+                bf16x8 ka[2][QB];
 #pragma unroll
-            for (int x = 0; x < KS; ++x)
-                sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + x * 32), qf[x],
-                                                                sc[kt], 0, 0, 0);
+                for (int i = 0; i < QB; ++i)
+                    if (x0 + i < KS)
+#pragma unroll
+                        for (int kt = 0; kt < 2; ++kt)
+                            ka[kt][i] = *reinterpret_cast<const bf16x8*>(krow + kt * 16 * kstride + (x0 + i) * 32);
+#pragma unroll
+                for (int i = 0; i < QB; ++i)
+                    if (x0 + i < KS)
+#pragma unroll
+                        for (int kt = 0; kt < 2; ++kt)
+                            sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kt][i], qf[x0 + i], sc[kt], 0, 0, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * QB, 0);      // the batch's LDS reads, then its products
+                __builtin_amdgcn_sched_group_barrier(0x008, 2 * QB, 0);
+            }
         }
         // the lane holds the keys c0 + 16 kt + 4 g + r of its column; scores in units of log 2, so that
         // every exponential is one instruction
@@ -202,16 +227,27 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
         l_run = fmaf(l_run, alpha, sum);
         m_run = m_new;
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
-        // O^T += C^T . P^T
+        // O^T += C^T . P^T, the operands again a batch at a time
+        if (rescale)
 #pragma unroll
-        for (int d = 0; d < NH; ++d)
-            if ((half * NH + d) * 16 < R) {
-                if (rescale)
+            for (int d = 0; d < NH; ++d)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[d][r] *= alpha;
-                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt_lds + ((half * NH + d) * 16 + col) * LM_VSTRIDE + 8 * g);
-                o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[d], 0, 0, 0);
+                for (int r = 0; r < 4; ++r) o[d][r] *= alpha;
+        {
+            constexpr int PB = NH < 8 ? NH : 8;
+            const bf16* vrow = vt_lds + ((half * NH) * 16 + col) * LM_VSTRIDE + 8 * g;
+#pragma unroll
+            for (int d0 = 0; d0 < NH; d0 += PB) {
+                bf16x8 va[PB];
+#pragma unroll
+                for (int i = 0; i < PB; ++i)
+                    if ((half * NH + d0 + i) * 16 < R) va[i] = *reinterpret_cast<const bf16x8*>(vrow + (d0 + i) * 16 * LM_VSTRIDE);
+#pragma unroll
+                for (int i = 0; i < PB; ++i)
+                    if ((half * NH + d0 + i) * 16 < R)
+                        o[d0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[i], pb, o[d0 + i], 0, 0, 0);
             }
+        }
     }
     if (!wave_live || !q_live) return;
     // the lane holds the entries 16 d + 4 g + r of its column
@@ -288,7 +324,7 @@ LC_API int lc_latent_bf16_supported(int R, int rot) {
 LC_API int lc_latent_bf16_splits(int workgroups, int max_keys) {
     if (workgroups <= 0) return 1;
     const int stages = (max_keys + LM_STAGE - 1) / LM_STAGE;
-    int want = (2 * device_cus() + workgroups - 1) / workgroups;      // two workgroups a CU
+    int want = (device_cus() + workgroups - 1) / workgroups;          // one workgroup a CU: a CU holds no more
     if (want > stages / 2) want = stages / 2;                          // two stages a share at least
     if (want > 64) want = 64;
     return want < 2 ? 1 : want;

@@ -150,3 +150,22 @@ def test_greedy_generation_through_the_scheduler(monkeypatch):
     assert got == [plain_pubodra.greedy(cfg, weights, p, 5) for p in prompts]
     engine.runner.cache.check()
     assert not engine.runner.cache.requests
+
+
+def test_latent_attention_planner():
+    """Tiles of up to 16 tokens of one request, a lone token a tile of its own, the tiles that see the
+    most keys first; sizes follow from the batch's make-up alone."""
+    from lucciola_amd.engine.batch import HostLayout
+    from lucciola_amd.kernels import ops
+    layout = HostLayout(num_requests=4, num_tokens=1 + 40 + 1 + 16, q_start=[0, 1, 41, 42, 58],
+                        first_position=[299, 0, 7, 100], block_size=16, single=False)
+    arrays, info = ops.plan_latent_attention(layout)
+    tiles = arrays["tiles"].tolist()
+    assert info == {"any_portion": True, "num_tiles": 6}
+    assert sorted(tiles) == sorted([[0, 1, 0, 299], [1, 16, 1, 0], [17, 16, 1, 16], [33, 8, 1, 32], [41, 1, 2, 7],
+                                    [42, 16, 3, 100]])
+    ends = [t[3] + t[1] for t in tiles]
+    assert ends == sorted(ends, reverse=True) and tiles[0] == [0, 1, 0, 299]
+    single = HostLayout(3, 3, [0, 1, 2, 3], [5, 50, 9], 16, True)
+    arrays, info = ops.plan_latent_attention(single)
+    assert info["any_portion"] is False and arrays["tiles"].shape == (3, 4)
