@@ -351,7 +351,7 @@ def design_configs(name, routed):
     mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
              "mask": {"size": 4096},
              "rot": {"base": 1000000.0, "dims": 64,
-                     "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+                     "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     dense = {"kind": "dense", "ff": ff}
     # the routed layer moves as many weights per token as the dense one: 4 of 32 experts of ff / 4
     moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}}

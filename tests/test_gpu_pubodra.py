@@ -89,7 +89,7 @@ def test_grouped_product_over_heads(dtype, rows, G, N, K, pad_x, gap):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,E,top,H,I", [(1, 4, 4, 20, 12), (9, 5, 1, 33, 17), (70, 12, 3, 64, 40), (300, 3, 2, 48, 64)])
+@pytest.mark.parametrize("T,E,top,H,I", [(1, 4, 4, 20, 12), (9, 5, 1, 33, 17), (70, 11, 3, 64, 40), (300, 3, 2, 48, 64)])
 def test_routed_experts(dtype, T, E, top, H, I):
     g = torch.Generator().manual_seed(T + E)
     x = torch.randn(T, H, generator=g).to(dtype)
