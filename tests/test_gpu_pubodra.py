@@ -424,3 +424,32 @@ def test_matrix_core_path_is_the_one_that_serves():
     compare(fast, cfg, weights, prompts, TOL["bfloat16"], refs)
     compare(slow, cfg, weights, prompts, TOL["bfloat16"], refs)
     assert any(not torch.equal(fast[k], slow[k]) for k in fast), "both runs took the same kernel"
+
+
+def test_command_line(tmp_path):
+    """A model folder made from a configuration and a seed, then greedy tokens through
+    ``python -m lucciola_amd``: the architecture is found by config.json alone."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = pubodra_configs.ALL["A"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(dict(cfg, initializer_range=0.2)))
+    folder = str(tmp_path / "model")
+    run = [sys.executable, "-m", "lucciola_amd"]
+    made = subprocess.run(run + ["--random-config", str(config_file), "--seed", "4", "--write-model", folder],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert made.returncode == 0, made.stderr[-2000:]
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = [[3, 17, 150, 9], [88] * 30 + [5, 6]]
+    proc = subprocess.run(run + ["--model", folder, "--dtype", "float32", "--max-new-tokens", "6", "--max-blocks", "64",
+                                 "--block-size", str(page), "--max-tokens-per-step", "12"]
+                          + [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()]
+    assert got == [plain_pubodra.greedy(cfg, weights, p, 6) for p in prompts]
