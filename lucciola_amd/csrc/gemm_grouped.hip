@@ -197,11 +197,11 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_kernel(GroupedArgs a) {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int GH_K = 32, GH_STRIDE = GH_K + 8;
 
-template <typename TO, int BM, int WM, int WN>
+template <typename TO, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(256, 2) void gemm_grouped_bf16_kernel(GroupedArgs a) {
     static_assert(WM * WN == 4, "four waves");
-    constexpr int BN = GG_N;
     constexpr int TM = BM / 16 / WM, TN = BN / 16 / WN;
+    constexpr int XL = (BM * 4 + 255) / 256, WL = (BN * 4 + 255) / 256;   // 16-byte pieces a thread brings a step
     __shared__ __align__(16) bf16 xs[2][BM][GH_STRIDE];
     __shared__ __align__(16) bf16 ws[2][BN][GH_STRIDE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
@@ -227,25 +227,42 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_bf16_kernel(GroupedArgs a
     const bf16* x = reinterpret_cast<const bf16*>(a.x) + (size_t)grp * a.x_group;
     const bf16* w = reinterpret_cast<const bf16*>(a.w) + (size_t)grp * N * K;
     const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
-    // loader: a thread brings one 16-byte piece (8 k) of a row of w and, where it has one, of x
+    // loader: a thread brings 16-byte pieces (8 k) of rows of x and of w, 64 rows apart
     const int lrow = tid >> 2, lk = (tid & 3) * 8;
-    const bool xlive = lrow < BM && r0 + lrow < r_end;
-    const bool wlive = n0 + lrow < N;
-    const int m_src = xlive ? r0 + lrow : r0;
-    const bf16* xrow = x + (size_t)(a.gather ? a.gather[m_src] : m_src) * a.ldx + lk;
-    const bf16* wrow = w + (size_t)(wlive ? n0 + lrow : 0) * K + lk;
+    bool xlive[XL], wlive[WL];
+    const bf16* xrow[XL];
+    const bf16* wrow[WL];
+#pragma unroll
+    for (int u = 0; u < XL; ++u) {
+        const int row = lrow + 64 * u;
+        xlive[u] = row < BM && r0 + row < r_end;
+        const int m_src = xlive[u] ? r0 + row : r0;
+        xrow[u] = x + (size_t)(a.gather ? a.gather[m_src] : m_src) * a.ldx + lk;
+    }
+#pragma unroll
+    for (int u = 0; u < WL; ++u) {
+        const int row = lrow + 64 * u;
+        wlive[u] = row < BN && n0 + row < N;
+        wrow[u] = w + (size_t)(wlive[u] ? n0 + row : 0) * K + lk;
+    }
     bf16x8 zero;
 #pragma unroll
     for (int i = 0; i < 8; ++i) zero[i] = static_cast<bf16>(0.f);
-    bf16x8 xr = zero, wr = zero;
+    bf16x8 xr[XL], wr[WL];
     auto fetch = [&](int k0) {
         const bool in = k0 + lk < K;                // K % 8 == 0: a piece is whole or absent
-        xr = (xlive && in) ? *reinterpret_cast<const bf16x8*>(xrow + k0) : zero;
-        wr = (wlive && in) ? *reinterpret_cast<const bf16x8*>(wrow + k0) : zero;
+#pragma unroll
+        for (int u = 0; u < XL; ++u) xr[u] = (xlive[u] && in) ? *reinterpret_cast<const bf16x8*>(xrow[u] + k0) : zero;
+#pragma unroll
+        for (int u = 0; u < WL; ++u) wr[u] = (wlive[u] && in) ? *reinterpret_cast<const bf16x8*>(wrow[u] + k0) : zero;
     };
     auto put = [&](int stage) {
-        if (lrow < BM) *reinterpret_cast<bf16x8*>(&xs[stage][lrow][lk]) = xr;
-        *reinterpret_cast<bf16x8*>(&ws[stage][lrow][lk]) = wr;
+#pragma unroll
+        for (int u = 0; u < XL; ++u)
+            if (lrow + 64 * u < BM) *reinterpret_cast<bf16x8*>(&xs[stage][lrow + 64 * u][lk]) = xr[u];
+#pragma unroll
+        for (int u = 0; u < WL; ++u)
+            if (lrow + 64 * u < BN) *reinterpret_cast<bf16x8*>(&ws[stage][lrow + 64 * u][lk]) = wr[u];
     };
     floatx4 acc[TM][TN];
 #pragma unroll
@@ -292,23 +309,25 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_bf16_kernel(GroupedArgs a
 }
 
 template <typename TO>
-static int launch_grouped_bf16(const GroupedArgs& a, int max_tiles, int small, hipStream_t stream) {
-    const int nb = (a.N + GG_N - 1) / GG_N;
-    if (small) {
-        dim3 grid(nb, a.row_start ? max_tiles : (a.M + 15) / 16, a.row_start ? 1 : a.G);
-        gemm_grouped_bf16_kernel<TO, 16, 1, 4><<<grid, 256, 0, stream>>>(a);
+static int launch_grouped_bf16(const GroupedArgs& a, int max_tiles, int tile_rows, hipStream_t stream) {
+    if (tile_rows == 16) {
+        dim3 grid((a.N + 63) / 64, a.row_start ? max_tiles : (a.M + 15) / 16, a.row_start ? 1 : a.G);
+        gemm_grouped_bf16_kernel<TO, 16, 64, 1, 4><<<grid, 256, 0, stream>>>(a);
+    } else if (tile_rows == 128) {
+        dim3 grid((a.N + 127) / 128, a.row_start ? max_tiles : (a.M + 127) / 128, a.row_start ? 1 : a.G);
+        gemm_grouped_bf16_kernel<TO, 128, 128, 2, 2><<<grid, 256, 0, stream>>>(a);
     } else {
-        dim3 grid(nb, a.row_start ? max_tiles : (a.M + 63) / 64, a.row_start ? 1 : a.G);
-        gemm_grouped_bf16_kernel<TO, 64, 2, 2><<<grid, 256, 0, stream>>>(a);
+        dim3 grid((a.N + 63) / 64, a.row_start ? max_tiles : (a.M + 63) / 64, a.row_start ? 1 : a.G);
+        gemm_grouped_bf16_kernel<TO, 64, 64, 2, 2><<<grid, 256, 0, stream>>>(a);
     }
     LC_LAUNCH_CHECK("gemm_grouped_bf16");
     return 0;
 }
 
 template <typename TX, typename TW, typename TO>
-static int launch_grouped(const GroupedArgs& a, int max_tiles, int small, hipStream_t stream) {
+static int launch_grouped(const GroupedArgs& a, int max_tiles, int tile_rows, hipStream_t stream) {
     const int nb = (a.N + GG_N - 1) / GG_N;
-    if (small) {
+    if (tile_rows == 16) {
         dim3 grid(nb, a.row_start ? max_tiles : (a.M + 15) / 16, a.row_start ? 1 : a.G);
         gemm_grouped_kernel<TX, TW, TO, 16, 1, 4><<<grid, 256, 0, stream>>>(a);
     } else {
@@ -331,15 +350,19 @@ LC_API int lc_gemm_grouped_fast(int on) {
     return before;
 }
 
-// Rows of a tile: 16 where `small`, else 64; the lists' tile_start must have been made for it.
-LC_API int lc_gemm_grouped_tile_rows(int small) { return small ? 16 : 64; }
+// Whether tiles of `tile_rows` rows exist for these operand types (16 and 64: always; 128: the
+// bfloat16 kernel only).  The lists' tile_start must have been made for the size that is asked for.
+LC_API int lc_gemm_grouped_takes_tile(int tile_rows, int x_dt, int w_dt) {
+    if (tile_rows == 16 || tile_rows == 64) return 1;
+    return tile_rows == 128 && x_dt == DT_BF16 && w_dt == DT_BF16 && g_grouped_fast ? 1 : 0;
+}
 
 // x, gate: dtype x_dt; w: w_dt; out: out_dt.  lists: row_start and tile_start [G + 1] on the
 // device, max_tiles the grid's room; M then is the number of sorted rows.  heads: both null.
 LC_API int lc_gemm_grouped(const void* x, int x_dt, long long ldx, long long x_group, const void* w, int w_dt,
                            void* out, int out_dt, long long ldo, long long out_group, int M, int N, int K, int G,
                            const int* gather, const int* row_start, const int* tile_start, int max_tiles,
-                           int small, int epilogue, const void* gate, long long ldg, long long gate_group,
+                           int tile_rows, int epilogue, const void* gate, long long ldg, long long gate_group,
                            hipStream_t stream) {
     LC_CHECK(M >= 0 && N > 0 && K > 0 && G > 0, "grouped product: bad sizes M=%d N=%d K=%d G=%d", M, N, K, G);
     if (M == 0) return 0;
@@ -349,23 +372,26 @@ LC_API int lc_gemm_grouped(const void* x, int x_dt, long long ldx, long long x_g
     LC_CHECK(!row_start || max_tiles > 0, "grouped product: no room for tiles");
     LC_CHECK(epilogue >= ACT_NONE && epilogue <= ACT_SIGMOID_GATE, "grouped product: unknown epilogue %d", epilogue);
     LC_CHECK(epilogue != ACT_SIGMOID_GATE || gate, "grouped product: no gates");
+    LC_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped product: tiles of %d rows", tile_rows);
     LC_CHECK(G <= 65535 && (row_start ? max_tiles : (M + 15) / 16) <= 65535, "grouped product: too many tiles");
     GroupedArgs a{x, ldx, x_group, w, out, ldo, out_group, M, N, K, G, gather, row_start, tile_start,
                   epilogue, gate, ldg, gate_group};
     // bfloat16 operands whose pieces of 8 are whole and aligned: the bfloat16 matrix instruction
     if (x_dt == DT_BF16 && w_dt == DT_BF16 && K % 8 == 0 && ldx % 8 == 0 && x_group % 8 == 0 &&
         (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && g_grouped_fast) {
-        if (out_dt == DT_BF16) return launch_grouped_bf16<bf16>(a, max_tiles, small, stream);
-        if (out_dt == DT_F32) return launch_grouped_bf16<float>(a, max_tiles, small, stream);
+        if (out_dt == DT_BF16) return launch_grouped_bf16<bf16>(a, max_tiles, tile_rows, stream);
+        if (out_dt == DT_F32) return launch_grouped_bf16<float>(a, max_tiles, tile_rows, stream);
     }
+    LC_CHECK(tile_rows != 128 || !row_start, "grouped product: lists made for tiles of 128 rows need whole aligned bfloat16 pieces");
+    if (tile_rows == 128) tile_rows = 64;
     const int key = x_dt * 4 + w_dt * 2 + out_dt;
     switch (key) {
-        case 0: return launch_grouped<float, float, float>(a, max_tiles, small, stream);
-        case 2: return launch_grouped<float, bf16, float>(a, max_tiles, small, stream);
-        case 4: return launch_grouped<bf16, float, float>(a, max_tiles, small, stream);
-        case 5: return launch_grouped<bf16, float, bf16>(a, max_tiles, small, stream);
-        case 6: return launch_grouped<bf16, bf16, float>(a, max_tiles, small, stream);
-        case 7: return launch_grouped<bf16, bf16, bf16>(a, max_tiles, small, stream);
+        case 0: return launch_grouped<float, float, float>(a, max_tiles, tile_rows, stream);
+        case 2: return launch_grouped<float, bf16, float>(a, max_tiles, tile_rows, stream);
+        case 4: return launch_grouped<bf16, float, float>(a, max_tiles, tile_rows, stream);
+        case 5: return launch_grouped<bf16, float, bf16>(a, max_tiles, tile_rows, stream);
+        case 6: return launch_grouped<bf16, bf16, float>(a, max_tiles, tile_rows, stream);
+        case 7: return launch_grouped<bf16, bf16, bf16>(a, max_tiles, tile_rows, stream);
         default:
             LC_CHECK(false, "grouped product: unsupported dtypes x=%d w=%d out=%d", x_dt, w_dt, out_dt);
     }

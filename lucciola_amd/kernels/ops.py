@@ -75,6 +75,7 @@ _SIGNATURES = {
     "lc_activation": "piiqp",
     "lc_gemm_grouped": "piqqpipiqqiiiipppiiipqqp",
     "lc_gemm_grouped_fast": "i",
+    "lc_gemm_grouped_takes_tile": "iii",
     "lc_latent_prepare": "piqiiiiipfppiipppp",
     "lc_latent_attention": "piiiiippppiifipp",
     "lc_latent_bf16_supported": "ii",
@@ -956,6 +957,16 @@ def _check_strided(s: Strided, what: str, rows: int, groups: int, width: int, dt
                           f"and {rows} rows do not fit {tuple(s.tensor.shape)}")
 
 
+def _grouped_tile(rows: int, N: int, x: torch.Tensor, w: torch.Tensor) -> int:
+    """Rows of a grouped product's tiles, for ``rows`` rows a group: 16 for a step of few tokens, 128
+    (by 128 columns) where the rows and columns are many and the operands take the bfloat16 kernel."""
+    if rows <= 16:
+        return 16
+    if rows >= 256 and N >= 128 and library().lc_gemm_grouped_takes_tile(128, _dt(x), _dt(w)):
+        return 128
+    return 64
+
+
 def grouped_gemm(x: Strided, w: torch.Tensor, out: Strided, rows: int, gate: Optional[Strided] = None,
                  activation: Optional[str] = None) -> None:
     """For every group g: ``out_g = x_g . w[g]^T`` over the first ``rows`` rows, with ``w`` [G, N, K], x_g
@@ -976,7 +987,7 @@ def grouped_gemm(x: Strided, w: torch.Tensor, out: Strided, rows: int, gate: Opt
         return
     _call("lc_gemm_grouped", x.pointer(), _dt(x.tensor), x.tensor.shape[1], x.group, _ptr(w), _dt(w),
           out.pointer(), _dt(out.tensor), out.tensor.shape[1], out.group, rows, N, K, G, None, None, None, 0,
-          1 if rows <= 16 else 0, epilogue, gate.pointer() if gate is not None else None,
+          _grouped_tile(rows, N, x.tensor, w), epilogue, gate.pointer() if gate is not None else None,
           gate.tensor.shape[1] if gate is not None else 0, gate.group if gate is not None else 0, _stream())
 
 
@@ -1125,14 +1136,16 @@ class Routing:
     sorted_token: torch.Tensor
     entry_row: torch.Tensor
     experts: int
-    small_tiles: bool
+    tile: int                   # rows of a tile of the sorted rows: what tile_start counts
     max_tiles: int
 
 
-def moe_route(logits: torch.Tensor, top: int, renormalise: bool = True, eps: float = 1e-20) -> Routing:
+def moe_route(logits: torch.Tensor, top: int, renormalise: bool = True, eps: float = 1e-20,
+              large_tiles: bool = False) -> Routing:
     """From the router's float32 ``logits`` [T, E]: softmax over all experts, the ``top`` largest scores of
     every token, divided by their sum + ``eps`` where ``renormalise``, and the lists that sort the
-    (token, choice) pairs by expert for :func:`moe_experts`."""
+    (token, choice) pairs by expert for :func:`moe_experts`.  ``large_tiles``: the experts' products will
+    take tiles of 128 rows (:func:`moe_large_tiles` says whether they do)."""
     _need(logits, "router logits", torch.float32, 2)
     T, E = logits.shape
     dev = logits.device
@@ -1140,14 +1153,24 @@ def moe_route(logits: torch.Tensor, top: int, renormalise: bool = True, eps: flo
     weights = torch.empty((T, top), dtype=torch.float32, device=dev)
     _call("lc_moe_route", _ptr(logits), T, E, top, 1 if renormalise else 0, float(eps), _ptr(ids), _ptr(weights),
           _stream())
-    small = T * top <= 16 * E       # few rows an expert: tiles of 16 rows, else of 64
-    tile = 16 if small else 64
+    # few rows an expert: tiles of 16 rows; many, and the caller's products take them: of 128; else of 64
+    tile = 16 if T * top <= 16 * E else 128 if (large_tiles and T * top >= 192 * E) else 64
     lists = torch.empty((2 * (E + 1) + 2 * T * top,), dtype=torch.int32, device=dev)
     row_start, tile_start = lists[:E + 1], lists[E + 1:2 * (E + 1)]
     sorted_token, entry_row = lists[2 * (E + 1):2 * (E + 1) + T * top], lists[2 * (E + 1) + T * top:]
     _call("lc_moe_lists", _ptr(ids), T, top, E, tile, _ptr(row_start), _ptr(tile_start), _ptr(sorted_token),
           _ptr(entry_row), _stream())
-    return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, small, (T * top) // tile + E)
+    return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, tile, (T * top) // tile + E)
+
+
+def moe_large_tiles(x_dtype: torch.dtype, up: torch.Tensor, down: torch.Tensor) -> bool:
+    """Whether both of the experts' products (weights ``up`` [E, I, H], ``down`` [E, H, I]) can run in tiles
+    of 128 rows: bfloat16 operands whose rows are whole 16-byte pieces, 128 columns at least."""
+    if x_dtype != torch.bfloat16 or up.dtype != torch.bfloat16 or down.dtype != torch.bfloat16:
+        return False
+    (_, I, H) = up.shape
+    return bool(I % 8 == 0 and H % 8 == 0 and I >= 128 and H >= 128
+                and library().lc_gemm_grouped_takes_tile(128, DT_BF16, DT_BF16))
 
 
 def moe_experts(x: torch.Tensor, w: torch.Tensor, routing: Routing, out_dtype: torch.dtype,
@@ -1165,7 +1188,7 @@ def moe_experts(x: torch.Tensor, w: torch.Tensor, routing: Routing, out_dtype: t
     if rows:
         _call("lc_gemm_grouped", _ptr(x), _dt(x), K, 0, _ptr(w), _dt(w), _ptr(out), _dt(out), N, 0, rows, N, K, E,
               _ptr(routing.sorted_token if gather else None), _ptr(routing.row_start), _ptr(routing.tile_start),
-              routing.max_tiles, 1 if routing.small_tiles else 0, ACTIVATIONS[activation] if activation else 0,
+              routing.max_tiles, routing.tile, ACTIVATIONS[activation] if activation else 0,
               None, 0, 0, _stream())
     return out
 

@@ -123,10 +123,12 @@ class RoutedMLP(Part):
         self.up = stack_rows([tensors[f"experts.{k}.up"] for k in range(self.E)]).view(self.E, self.I, self.H)
         self.down = stack_rows([tensors[f"experts.{k}.down"] for k in range(self.E)]).view(self.E, self.H, self.I)
         self.dtype = ctx.dtype
+        self.large_tiles = ctx.device.type == "cuda" and ops.moe_large_tiles(ctx.dtype, self.up, self.down)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = ops.gemm(x, self.router, torch.float32)
-        routing = ops.moe_route(logits, self.top, self.renormalise, self.renormalise_eps)
+        routing = ops.moe_route(logits, self.top, self.renormalise, self.renormalise_eps,
+                                large_tiles=self.large_tiles)
         hidden = ops.moe_experts(x, self.up, routing, self.dtype, activation=self.activation, gather=True)
         y = ops.moe_experts(hidden, self.down, routing, torch.float32)
         return ops.moe_combine(y, routing, self.dtype)

@@ -232,7 +232,7 @@ class _Routing:
     pass
 
 
-def moe_route(logits, top, renormalise=True, eps=1e-20):
+def moe_route(logits, top, renormalise=True, eps=1e-20, large_tiles=False):
     s = torch.softmax(logits.to(F64), dim=-1)
     picked, ids = torch.topk(s, top, dim=-1)
     if renormalise:

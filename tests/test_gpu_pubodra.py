@@ -70,7 +70,8 @@ def test_stream_add_and_activations():
 @pytest.mark.parametrize("rows,G,N,K,pad_x,gap", [(1, 3, 21, 7, 5, 2), (16, 2, 64, 32, 5, 2), (77, 5, 18, 300, 5, 2),
                                                   (130, 1, 100, 9, 5, 2),
                                                   # whole 16-byte pieces: in bfloat16 the bfloat16 matrix instruction
-                                                  (3, 4, 96, 32, 8, 8), (70, 3, 40, 136, 16, 0), (200, 2, 130, 512, 0, 64)])
+                                                  (3, 4, 96, 32, 8, 8), (70, 3, 40, 136, 16, 0), (200, 2, 130, 512, 0, 64),
+                                                  (300, 3, 200, 264, 0, 8)])     # many rows: tiles of 128 x 128
 def test_grouped_product_over_heads(dtype, rows, G, N, K, pad_x, gap):
     g = torch.Generator().manual_seed(rows * 7 + G)
     pad_o = 3
@@ -89,7 +90,8 @@ def test_grouped_product_over_heads(dtype, rows, G, N, K, pad_x, gap):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,E,top,H,I", [(1, 4, 4, 20, 12), (9, 5, 1, 33, 17), (70, 11, 3, 64, 40), (300, 3, 2, 48, 64)])
+@pytest.mark.parametrize("T,E,top,H,I", [(1, 4, 4, 20, 12), (9, 5, 1, 33, 17), (70, 11, 3, 64, 40), (300, 3, 2, 48, 64),
+                                         (700, 3, 2, 136, 200)])      # many rows an expert: tiles of 128
 def test_routed_experts(dtype, T, E, top, H, I):
     g = torch.Generator().manual_seed(T + E)
     x = torch.randn(T, H, generator=g).to(dtype)
@@ -99,7 +101,9 @@ def test_routed_experts(dtype, T, E, top, H, I):
     want = reference_ops.moe_combine(
         reference_ops.moe_experts(reference_ops.moe_experts(x, up, r_ref, dtype, "relu_squared", True), down, r_ref,
                                   torch.float32), r_ref, dtype)
-    r = ops.moe_route(logits.to(DEV), top, True, 1e-20)
+    large = ops.moe_large_tiles(dtype, up.to(DEV), down.to(DEV))
+    r = ops.moe_route(logits.to(DEV), top, True, 1e-20, large_tiles=large)
+    assert r.tile == (128 if (large and T * top >= 192 * E) else 16 if T * top <= 16 * E else 64)
     assert torch.equal(r.ids.cpu(), r_ref.ids), "chosen experts"
     assert torch.allclose(r.weights.cpu(), r_ref.weights, atol=1e-6)
     starts = r.row_start.cpu().tolist()
