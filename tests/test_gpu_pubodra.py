@@ -71,7 +71,7 @@ def test_stream_add_and_activations():
                                                   (130, 1, 100, 9, 5, 2),
                                                   # whole 16-byte pieces: in bfloat16 the bfloat16 matrix instruction
                                                   (3, 4, 96, 32, 8, 8), (70, 3, 40, 136, 16, 0), (200, 2, 130, 512, 0, 64),
-                                                  (300, 3, 200, 264, 0, 8)])     # many rows: tiles of 128 x 128
+                                                  (1300, 16, 1100, 40, 0, 8)])     # many tiles: 128 x 128
 def test_grouped_product_over_heads(dtype, rows, G, N, K, pad_x, gap):
     g = torch.Generator().manual_seed(rows * 7 + G)
     pad_o = 3
