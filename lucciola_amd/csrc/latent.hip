@@ -19,7 +19,7 @@ namespace lc {
 constexpr int LA_THREADS = 256;
 constexpr int LA_HEADS = 4;       // heads a workgroup serves together: one wave each for the softmax
 constexpr int LA_KEYS = 64;       // keys of a chunk
-constexpr int LA_DIMS = 4;        // output entries a thread sums: R <= LA_THREADS * LA_DIMS
+constexpr int LA_DIMS = 8;        // output entries a thread sums: R <= LA_THREADS * LA_DIMS
 
 // ------------------------------------------------------------------------------ prologue
 // One workgroup per token.  From the row [q heads | c' | k_r | ...] of the fused projection:

@@ -117,7 +117,7 @@ def test_routed_experts(dtype, T, E, top, H, I):
 @pytest.mark.parametrize("heads,dim,rot,rank,rd,pairing,page,window",
                          [(3, 7, 10, 21, 6, "interleaved", 8, 17), (4, 16, 8, 32, 8, "interleaved", 4, 0),
                           (5, 0, 12, 40, 12, "half", 16, 70), (1, 5, 0, 9, 0, "interleaved", 2, 3),
-                          (9, 8, 16, 300, 16, "interleaved", 16, 130)])
+                          (9, 8, 16, 300, 16, "interleaved", 16, 130), (2, 4, 4, 1100, 4, "interleaved", 16, 50)])
 def test_latent_attention_kernels(dtype, heads, dim, rot, rank, rd, pairing, page, window):
     """Two requests of unequal length written to scattered pages in two portions each, then read."""
     g = torch.Generator().manual_seed(heads * 100 + rank)
