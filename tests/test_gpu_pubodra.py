@@ -28,8 +28,10 @@ def case(key):
     return _cache[key]
 
 
-def close(got, want, dtype, what):
-    tol = 3e-6 if dtype == torch.float32 else 1.2e-2
+def close(got, want, dtype, what, terms=1):
+    """``terms``: how many times longer the sums are than the few hundred terms the bounds are set for
+    (float32 rounding grows with the length of a sum)."""
+    tol = (3e-6 if dtype == torch.float32 else 1.2e-2) * max(1.0, terms) ** 0.5
     err = float((got.double() - want.double()).abs().max() / want.double().abs().max().clamp_min(1e-9))
     assert err < tol, f"{what}: relative error {err:.3e}"
 
@@ -158,7 +160,7 @@ def test_latent_attention_kernels(dtype, heads, dim, rot, rank, rd, pairing, pag
         close(outs[1][0], outs[0][0], dtype, "rotated queries")
         close(caches[1].cpu(), caches[0], dtype, "cache rows")
         caches[1].copy_(caches[0])        # the same rows on both sides for the attention itself
-        close(outs[1][1], outs[0][1], dtype, "latent attention")
+        close(outs[1][1], outs[0][1], dtype, "latent attention", terms=(rank + rot) / 300)
 
 
 def test_rotary_table_stretched():
