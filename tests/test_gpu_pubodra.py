@@ -459,3 +459,21 @@ def test_command_line(tmp_path):
     assert proc.returncode == 0, proc.stderr[-2000:]
     got = [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()]
     assert got == [plain_pubodra.greedy(cfg, weights, p, 6) for p in prompts]
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_generation_survives_preemption(ahead):
+    """With so few pages that running requests are preempted and recomputed (the windows give pages
+    back, full attention in one layer of B does not), every request's tokens are the plain
+    implementation's; also with the next step queued before this step's tokens are read."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = pubodra_configs.ALL["B"]
+    weights = random_weights(cfg, seed, std=0.2)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [9, 14, 6, 11], seed + 40).values())
+    tight = engine_for(cfg, weights, page, 9, "float32", max_tokens_per_step=12, max_seqs=4, run_ahead=ahead)
+    got = tight.generate(prompts, SamplingParams(max_new_tokens=20))
+    assert tight.scheduler.num_preemptions > 0
+    for prompt, tokens in zip(prompts, got):
+        assert tokens == plain_pubodra.greedy(cfg, weights, prompt, 20)
+    tight.runner.cache.check()
+    assert not tight.runner.cache.requests
