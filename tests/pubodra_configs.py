@@ -65,3 +65,39 @@ P_C = {
 
 ALL = {"A": (P_A, 4, 11), "B": (P_B, 8, 12), "C": (P_C, 16, 13)}
 STD = 0.05      # spread of the random weights: every branch moves the logits, and no router call is so close that bfloat16 flips it
+
+
+def random_configuration(seed):
+    """A configuration drawn at random: every size, the layers' order and kinds, the windows, the
+    rotary constants and the place of the repeated stretch."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([24, 40, 64, 72, 96, 128])
+    layers = []
+    for _ in range(rng.randint(1, 4)):
+        heads = rng.choice([1, 2, 3, 4, 6, 8])
+        dim = rng.choice([0, 4, 8, 12, 16, 32])
+        rot_dim = rng.choice([2, 4, 8, 16, 32] if dim else [4, 8, 16])
+        dims = rng.choice([rot_dim, rot_dim, max(2, rot_dim // 2)])
+        scaling = None
+        if rng.random() < 0.5:
+            scaling = {"factor": rng.choice([2.0, 4.0, 16.0]), "original": rng.choice([16, 64, 512]),
+                       "fast": rng.choice([8.0, 32.0]), "slow": rng.choice([1.0, 2.0])}
+        mixer = _mixer(heads, dim, rot_dim, rng.choice([4, 8, 12, 16, 32]), rng.choice([8, 16, 24, 32, 48, 56, 64, 80]),
+                       rng.choice([0.1, 0.2, 0.35]), rng.choice([None, 5, 16, 31, 64, 100]),
+                       base=rng.choice([100.0, 10000.0, 500000.0]), dims=dims, scaling=scaling)
+        kind = rng.random()
+        if kind < 0.2:
+            mlp = None
+        elif kind < 0.6:
+            mlp = _dense(rng.choice([32, 48, 100, 128]))
+        else:
+            experts = rng.choice([2, 4, 7, 16])
+            mlp = _moe(rng.choice([16, 24, 40, 64]), experts, rng.randint(1, min(4, experts)))
+        layers.append(_layer(mixer, mlp))
+    cfg = {"architecture": "Pubodra", "vocab": rng.choice([50, 257, 400]), "width": width,
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
+    if rng.random() < 0.7:
+        start = rng.randrange(len(layers))
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return cfg, rng.choice([4, 8, 16, 32])

@@ -477,3 +477,19 @@ def test_generation_survives_preemption(ahead):
         assert tokens == plain_pubodra.greedy(cfg, weights, prompt, 20)
     tight.runner.cache.check()
     assert not tight.runner.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(seed, dtype):
+    """Configurations drawn at random, requests in mixed steps with so few pages that they are used
+    again, against the plain implementation."""
+    cfg, page = pubodra_configs.random_configuration(seed)
+    weights = random_weights(cfg, 100 + seed, std=pubodra_configs.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [3, 120, 41, 77, 1, 150], seed)
+    refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.mixed(prompts, seed=seed)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    compare(replay(runner, steps), cfg, weights, prompts, TOL[dtype], refs)
+    assert not runner.cache.requests

@@ -169,3 +169,15 @@ def test_latent_attention_planner():
     single = HostLayout(3, 3, [0, 1, 2, 3], [5, 50, 9], 16, True)
     arrays, info = ops.plan_latent_attention(single)
     assert info["any_portion"] is False and arrays["tiles"].shape == (3, 4)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5])
+def test_random_configurations_on_the_host(monkeypatch, seed):
+    reference_ops.install(monkeypatch)
+    cfg, page = pubodra_configs.random_configuration(seed)
+    weights = random_weights(cfg, 100 + seed, std=pubodra_configs.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [3, 35, 18], seed)
+    steps = traces.mixed(prompts, seed=seed)
+    runner = make_runner(cfg, weights, page, traces.max_live_tokens(steps, page) // page, "float32", "cpu")
+    refs = {n: plain_pubodra.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    compare(replay(runner, steps), cfg, weights, prompts, 2e-5, refs)
