@@ -207,8 +207,11 @@ def load_declared(source: WeightSource, declared: Mapping[str, ParamDecl],
             stored_dtypes[name] = t.dtype
         target = kept_dtype(t.dtype, decl.role)
         # one copy: to the device first (as stored), then widen there if needed
+        here = t
         t = t.to(device=device, non_blocking=False)
         if t.dtype != target:
             t = t.to(target)
+        if t is here or t.data_ptr() == here.data_ptr():
+            t = t.clone()       # still the source's memory (a file's map, on the CPU): the source is closed after loading
         out[name] = t.contiguous()
     return out
