@@ -493,3 +493,32 @@ def test_random_configurations(seed, dtype):
     runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
     compare(replay(runner, steps), cfg, weights, prompts, TOL[dtype], refs)
     assert not runner.cache.requests
+
+
+@pytest.mark.parametrize("heads,rank,rot,page,window", [(16, 512, 64, 16, 0), (20, 64, 32, 16, 90), (3, 48, 8, 4, 37),
+                                                        (32, 208, 24, 32, 0), (1, 16, 0, 8, 5), (70, 64, 16, 16, 0)])
+def test_a_step_of_lone_tokens_on_the_matrix_cores(heads, rank, rot, page, window):
+    """A step of lone tokens only (after 299, 0, 64, 31 and 700 cached tokens), where a workgroup
+    serves up to 64 heads of one token, against the plain version; then with the keys shared out."""
+    from lucciola_amd.engine.batch import HostLayout, Plan
+    g = torch.Generator().manual_seed(heads * 3 + rank)
+    history = [299, 0, 64, 31, 700]
+    n_pages = sum(-(-(h + 1) // page) for h in history) + 2
+    order = torch.randperm(n_pages, generator=g).tolist()
+    width = max(-(-(h + 1) // page) for h in history)
+    block_table = torch.full((len(history), width), -1, dtype=torch.int32)
+    cache = (torch.randn(n_pages, page, rank + rot, generator=g) * 0.5).bfloat16()
+    for r, h in enumerate(history):
+        for b in range(-(-(h + 1) // page)):
+            block_table[r, b] = order.pop()
+    T = len(history)
+    tok_req = torch.arange(T, dtype=torch.int32)
+    positions = torch.tensor(history, dtype=torch.int32)
+    qa = torch.randn(T, heads * (rank + rot), generator=g).bfloat16()
+    arrays, info = ops.plan_latent_attention(HostLayout(T, T, list(range(T + 1)), history, page, True))
+    plan = Plan({k: torch.from_numpy(v).to(DEV) for k, v in arrays.items()}, info)
+    want = reference_ops.latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page, 0.2, window)
+    args = (qa.to(DEV), heads, rank, rot, tok_req.to(DEV), positions.to(DEV), block_table.to(DEV), cache.to(DEV), page,
+            0.2, window)
+    close(ops.latent_attention(*args, plan=plan, max_ctx=701).cpu(), want, torch.bfloat16, "lone tokens")
+    close(ops.latent_attention(*args, plan=plan, max_ctx=1 << 20).cpu(), want, torch.bfloat16, "lone tokens, many shares")
