@@ -139,3 +139,30 @@ class FixedState(CacheNeed):
 
     def start(self, storage, slot: int) -> None:
         storage[slot].zero_()
+
+
+@dataclass(frozen=True)
+class FixedStates(CacheNeed):
+    """Several float32 tensors of fixed shape per live request (a recurrent layer's matrix of
+    state and the last inputs of its short convolutions, say): a tuple of ``[max_seqs, *shape]``
+    tensors in the order of ``shapes``, indexed by the request's slot, all zeroed when a
+    request starts."""
+
+    shapes: Tuple[Tuple[int, ...], ...]
+
+    def bytes_per_request(self, dtype: torch.dtype) -> int:
+        total = 0
+        for shape in self.shapes:
+            count = 1
+            for n in shape:
+                count *= int(n)
+            total += 4 * count
+        return total
+
+    def allocate(self, layout: CacheLayout, dtype: torch.dtype, device):
+        return tuple(torch.zeros((layout.max_seqs,) + tuple(shape), dtype=torch.float32, device=device)
+                     for shape in self.shapes)
+
+    def start(self, storage, slot: int) -> None:
+        for tensor in storage:
+            tensor[slot].zero_()

@@ -85,6 +85,17 @@ _SIGNATURES = {
     "lc_moe_route": "piiiifppp",
     "lc_moe_lists": "piiiippppp",
     "lc_moe_combine": "pppiiipip",
+    "lc_layer_norm": "ppippfpppfpiiiiip",
+    "lc_embedding_sinusoid": "pppippiiifp",
+    "lc_gated_activation": "ppiiiip",
+    "lc_head_norm_write": "piiiiiiippfpppppiip",
+    "lc_general_delta_prepare": "piiiipppffppp",
+    "lc_gated_delta_prepare": "piiiiiippippfpppppp",
+    "lc_conv_tail_update": "piipiiippip",
+    "lc_delta_scan": "pppipppiiiiip",
+    "lc_head_gate_norm": "ppiipifiiiipip",
+    "lc_moe_route_logits": "pipiiippp",
+    "lc_moe_combine_shared": "pppiiipipiipip",
 }
 
 
@@ -286,7 +297,7 @@ class ProductShares:
 
 def value(t):
     """The tensor that ``t`` stands for (``t`` itself if it is one)."""
-    return t.value() if isinstance(t, (PendingProduct, ScaledRows, ProductShares)) else t
+    return t.value() if isinstance(t, (PendingProduct, ScaledRows, ProductShares, NormedBranch)) else t
 
 
 def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
@@ -1238,3 +1249,351 @@ def feed_tokens(ids: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor) 
         raise KernelError("feed_tokens: one source row per id")
     _call("lc_feed_tokens", _ptr(ids), _ptr(source), _ptr(sampled), _c_int(ids.shape[0]),
           _c_int(sampled.shape[0]), _stream())
+
+
+# ------------------------------------------------------------------------------ layer norm, position vector
+@dataclass
+class NormedBranch:
+    """A branch's output ``x`` [T, n] that is to pass a layer norm (``weight``, ``bias``, ``eps``)
+    before it is added to the residual stream.  :func:`layer_norm` takes it as the stream's pending
+    addition and does both in its kernel; anyone else gets the normed tensor from ``value()``."""
+
+    x: torch.Tensor
+    weight: torch.Tensor
+    bias: torch.Tensor
+    eps: float
+
+    def value(self) -> torch.Tensor:
+        return layer_norm_act(self.x, self.weight, self.bias, self.eps)
+
+
+def layer_norm(h: torch.Tensor, delta, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+               out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Layer norm ``(v - mean) / sqrt(var + eps) * weight + bias`` of the float32 residual stream ``h``
+    [T, n] with the pending addition ``delta`` taken in first (v = h + delta); ``delta`` may be a
+    :class:`NormedBranch`, which is normed with its own weights before it is added.  Without ``rows``:
+    ``h`` becomes v in place and every row is normed; with ``rows`` (int32 [R]): only those rows, ``h``
+    stays as it is."""
+    _need(h, "layer_norm h", torch.float32, 2)
+    _need(weight, "layer_norm weight", torch.float32, 1)
+    _need(bias, "layer_norm bias", torch.float32, 1)
+    T, n = h.shape
+    if weight.shape[0] != n or bias.shape[0] != n:
+        raise KernelError(f"layer_norm: weight and bias must have {n} entries")
+    post_w = post_b = None
+    post_eps = 0.0
+    if isinstance(delta, NormedBranch):
+        post_w, post_b, post_eps = delta.weight, delta.bias, delta.eps
+        _need(post_w, "layer_norm branch weight", torch.float32, 1)
+        _need(post_b, "layer_norm branch bias", torch.float32, 1)
+        if post_w.shape[0] != n or post_b.shape[0] != n:
+            raise KernelError(f"layer_norm: the branch's weight and bias must have {n} entries")
+        delta = delta.x
+    delta = value(delta)
+    if delta is not None:
+        _need(delta, "layer_norm delta", None, 2)
+        if tuple(delta.shape) != (T, n):
+            raise KernelError(f"layer_norm: delta {tuple(delta.shape)} does not match h {(T, n)}")
+    if rows is not None:
+        _need(rows, "layer_norm rows", torch.int32, 1)
+    R = T if rows is None else rows.shape[0]
+    out = torch.empty((R, n), dtype=out_dtype, device=h.device)
+    if R:
+        _call("lc_layer_norm", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(post_w),
+              _ptr(post_b), float(post_eps), _ptr(rows), _ptr(weight), _ptr(bias), float(eps), _ptr(out), _dt(out),
+              R, n, 1 if (rows is None and delta is not None) else 0, T, _stream())
+    return out
+
+
+def layer_norm_act(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float) -> torch.Tensor:
+    """Layer norm over the last dimension of an activation tensor, in its dtype."""
+    _need(x, "layer_norm_act x")
+    _need(weight, "layer_norm_act weight", torch.float32, 1)
+    _need(bias, "layer_norm_act bias", torch.float32, 1)
+    n = x.shape[-1]
+    if weight.shape[0] != n or bias.shape[0] != n:
+        raise KernelError(f"layer_norm_act: weight and bias must have {n} entries")
+    out = torch.empty_like(x)
+    rows = x.numel() // n
+    if rows:
+        _call("lc_layer_norm", None, _ptr(x), _dt(x), _ptr(weight), _ptr(bias), float(eps), None, None, None,
+              0.0, _ptr(out), _dt(out), rows, n, 0, rows, _stream())
+    return out
+
+
+def embedding_sinusoid(ids: torch.Tensor, table: torch.Tensor, positions: torch.Tensor,
+                       frequencies: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, H]: row ``ids[t]`` of ``table`` times ``scale`` plus the position vector of
+    ``positions[t]``: entry 2i is sin(p f_i), entry 2i + 1 cos(p f_i), ``frequencies`` float32 [ceil(H/2)]."""
+    _need(ids, "embedding ids", torch.int32, 1)
+    _need(positions, "embedding positions", torch.int32, 1)
+    _need(table, "embedding table", None, 2)
+    _need(frequencies, "embedding frequencies", torch.float32, 1)
+    T, (V, H) = ids.shape[0], table.shape
+    if positions.shape[0] != T or frequencies.shape[0] != (H + 1) // 2:
+        raise KernelError("embedding_sinusoid: one position per id and one frequency per pair of entries")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    if T:
+        _call("lc_embedding_sinusoid", _ptr(ids), _ptr(positions), _ptr(table), _dt(table), _ptr(frequencies),
+              _ptr(out), T, H, V, float(scale), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ gated activations
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gated_activation(gu: torch.Tensor, kind: str) -> torch.Tensor:
+    """``gu`` [T, 2 I] (gate columns, then up columns) -> act(gate) * up, [T, I]; float32 arithmetic."""
+    _need(gu, "gated_activation input", None, 2)
+    T, two_i = gu.shape
+    if two_i % 2:
+        raise KernelError("gated_activation: the input needs an even number of columns")
+    out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
+    if T:
+        _call("lc_gated_activation", _ptr(gu), _ptr(out), _dt(gu), T, two_i // 2, GATE_ACTIVATIONS[kind], _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ attention with heads in slots
+def attention_head_slot(size: int) -> int:
+    """The head size that the cache and the attention kernels use for heads of up to ``size`` entries:
+    the next size the matrix-core kernels are built for, else the next multiple of 16."""
+    for slot in (32, 64, 96, 128):
+        if size <= slot:
+            return slot
+    if size > 256:
+        raise KernelError(f"attention: heads of {size} entries are above the kernels' 256")
+    return -(-size // 16) * 16
+
+
+def head_norm_write(proj: torch.Tensor, nh: int, nkv: int, d: int, dv: int, slot: int,
+                    q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                    head_scale: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+    """From the raw projections ``proj`` [T, nh d + nkv d + nkv dv] (queries, keys, values; ``nkv`` = 0:
+    queries only): every q and k head divided by its root mean square over its ``d`` entries (eps
+    inside the root) and multiplied by its weight [d] (None: no norm), q head h also by
+    ``head_scale[h]``.  Returns q as [T, nh slot] (zeros behind the d entries); k and v go to the
+    cache slot ``slots[t]`` (negative: no write) as heads of ``slot`` entries, zeros behind theirs:
+    keys [pages, nkv, page_size, slot], values [pages, nkv, slot, page_size]."""
+    _need(proj, "head_norm_write proj", None, 2)
+    T = proj.shape[0]
+    if proj.shape[1] != nh * d + nkv * (d + dv):
+        raise KernelError(f"head_norm_write: proj has {proj.shape[1]} columns, expected {nh * d + nkv * (d + dv)}")
+    if d > slot or dv > slot:
+        raise KernelError(f"head_norm_write: heads of {d}/{dv} do not fit a slot of {slot}")
+    for wt, name in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
+        if wt is not None:
+            _need(wt, name, torch.float32, 1)
+            if wt.shape[0] != d:
+                raise KernelError(f"{name} has {wt.shape[0]} entries for head size {d}")
+    if head_scale is not None:
+        _need(head_scale, "head scale", torch.float32, 1)
+        if head_scale.shape[0] != nh:
+            raise KernelError(f"head scale has {head_scale.shape[0]} entries for {nh} heads")
+    if nkv and slots is not None and k_cache is not None:
+        _need(k_cache, "k cache", proj.dtype, 4)
+        _need(v_cache, "v cache", proj.dtype, 4)
+        _need(slots, "slots", torch.int32, 1)
+        _check_caches(k_cache, v_cache, nkv, page_size, slot)
+        if slots.shape[0] != T:
+            raise KernelError("slots do not match the tokens")
+    else:
+        k_cache = v_cache = slots = None
+    q = torch.empty((T, nh * slot), dtype=proj.dtype, device=proj.device)
+    if T:
+        _call("lc_head_norm_write", _ptr(proj), _dt(proj), T, nh, nkv, d, dv, slot, _ptr(q_weight), _ptr(k_weight),
+              float(eps), _ptr(head_scale), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(slots), page_size,
+              k_cache.shape[0] if k_cache is not None else 0, _stream())
+    return q
+
+
+# ------------------------------------------------------------------------------ delta rules
+DELTA_MAX_KEY = 256        # key channels of a head that the scan kernel holds (16 a lane, 16 lanes a column)
+CONV_MAX_TAPS = 16
+
+
+def check_delta_sizes(what: str, key_dim: int, value_dim: int, taps: int = 1) -> None:
+    if not 1 <= key_dim <= DELTA_MAX_KEY:
+        raise KernelError(f"{what}: a head's {key_dim} key channels are outside the scan kernel's 1..{DELTA_MAX_KEY}")
+    if value_dim < 1:
+        raise KernelError(f"{what}: a head needs value channels")
+    if not 1 <= taps <= CONV_MAX_TAPS:
+        raise KernelError(f"{what}: {taps} taps are outside the convolution kernel's 1..{CONV_MAX_TAPS}")
+
+
+def general_delta_prepare(proj: torch.Tensor, heads: int, dim: int, inner: int, decay_out: torch.Tensor,
+                          decay_bias: torch.Tensor, removal_bias: torch.Tensor, unit_eps: float,
+                          decay_scale: float):
+    """The scan's inputs of the generalized delta rule from the float32 projections ``proj``
+    [T, 5 n + inner], n = heads dim: columns r | k | v | gate | removal | decay_in.
+    decay = exp(-decay_scale sigmoid(decay_out tanh(decay_in) + decay_bias)), a = sigmoid(removal +
+    removal_bias), u = k / sqrt(sum k^2 + unit_eps) per head.  Returns ``coef`` float32 [5, T, n]
+    (decay, probe = u, removal = a u, write = k, read = r) and ``v`` float32 [T, n]."""
+    _need(proj, "general_delta proj", torch.float32, 2)
+    n = heads * dim
+    T = proj.shape[0]
+    if proj.shape[1] != 5 * n + inner:
+        raise KernelError(f"general_delta_prepare: proj has {proj.shape[1]} columns, expected {5 * n + inner}")
+    _need(decay_out, "decay_out", torch.float32, 2)
+    _need(decay_bias, "decay_bias", torch.float32, 1)
+    _need(removal_bias, "removal_bias", torch.float32, 1)
+    if tuple(decay_out.shape) != (n, inner) or decay_bias.shape[0] != n or removal_bias.shape[0] != n:
+        raise KernelError("general_delta_prepare: the decay's and the removal's tensors do not fit the heads")
+    coef = torch.empty((5, T, n), dtype=torch.float32, device=proj.device)
+    v = torch.empty((T, n), dtype=torch.float32, device=proj.device)
+    if T:
+        _call("lc_general_delta_prepare", _ptr(proj), T, heads, dim, inner, _ptr(decay_out), _ptr(decay_bias),
+              _ptr(removal_bias), float(unit_eps), float(decay_scale), _ptr(coef), _ptr(v), _stream())
+    return coef, v
+
+
+def gated_delta_prepare(proj: torch.Tensor, tail: torch.Tensor, taps: torch.Tensor, rate_log: torch.Tensor,
+                        rate_bias: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
+                        num_taps: int, unit_eps: float, tok_req: torch.Tensor, q_offsets: torch.Tensor,
+                        slot_ids: torch.Tensor):
+    """The scan's inputs of the gated delta rule from the float32 projections ``proj`` [T, C + nv + 2
+    heads]: columns q | k | v (the C = 2 kv_heads key_dim + heads value_dim channels that pass the
+    convolutions) | gate | beta | rate.  Channel c of token t becomes silu(sum_j taps[c, K - 1 - j] x[t -
+    j, c]); inputs from before the step come from ``tail`` [slots, K - 1, C] (the request's last K - 1
+    inputs, oldest first), zeros before the sequence's start.  q and k are made unit vectors per head
+    (q also times key_dim^-1/2); g = exp(-exp(rate_log) softplus(rate + rate_bias)), beta = sigmoid(beta).
+    Returns ``coef`` float32 [5, T, heads key_dim] (decay = g, probe = g k, removal = beta k, write = beta k,
+    read = q) and ``v`` float32 [T, heads value_dim]."""
+    _need(proj, "gated_delta proj", torch.float32, 2)
+    T = proj.shape[0]
+    C = 2 * kv_heads * key_dim + heads * value_dim
+    if proj.shape[1] != C + heads * value_dim + 2 * heads:
+        raise KernelError(f"gated_delta_prepare: proj has {proj.shape[1]} columns, expected "
+                          f"{C + heads * value_dim + 2 * heads}")
+    _need(taps, "conv taps", torch.float32, 2)
+    _need(tail, "conv tail", torch.float32, 3)
+    if tuple(taps.shape) != (C, num_taps) or tuple(tail.shape[1:]) != (num_taps - 1, C):
+        raise KernelError("gated_delta_prepare: taps or tail do not fit the channels")
+    _need(rate_log, "rate_log", torch.float32, 1)
+    _need(rate_bias, "rate_bias", torch.float32, 1)
+    _need(tok_req, "tok_req", torch.int32, 1)
+    _need(q_offsets, "q_offsets", torch.int32, 1)
+    _need(slot_ids, "slot_ids", torch.int32, 1)
+    if rate_log.shape[0] != heads or rate_bias.shape[0] != heads or tok_req.shape[0] != T:
+        raise KernelError("gated_delta_prepare: per-head vectors or the token map do not fit")
+    coef = torch.empty((5, T, heads * key_dim), dtype=torch.float32, device=proj.device)
+    v = torch.empty((T, heads * value_dim), dtype=torch.float32, device=proj.device)
+    if T:
+        _call("lc_gated_delta_prepare", _ptr(proj), T, heads, kv_heads, key_dim, value_dim, num_taps, _ptr(taps),
+              _ptr(tail), tail.shape[0], _ptr(rate_log), _ptr(rate_bias), float(unit_eps), _ptr(tok_req),
+              _ptr(q_offsets), _ptr(slot_ids), _ptr(coef), _ptr(v), _stream())
+    return coef, v
+
+
+def conv_tail_update(proj: torch.Tensor, tail: torch.Tensor, channels: int, num_taps: int,
+                     q_offsets: torch.Tensor, slot_ids: torch.Tensor, num_requests: int) -> None:
+    """After a step: ``tail`` [slots, K - 1, C] of every request of the batch becomes the last K - 1
+    rows of (its old tail, then the first ``channels`` columns of the request's rows of ``proj``)."""
+    _need(proj, "conv_tail_update proj", torch.float32, 2)
+    _need(tail, "conv tail", torch.float32, 3)
+    if num_taps <= 1 or num_requests == 0:
+        return
+    if tuple(tail.shape[1:]) != (num_taps - 1, channels) or proj.shape[1] < channels:
+        raise KernelError("conv_tail_update: the tail does not fit the channels")
+    if q_offsets.shape[0] != num_requests + 1 or slot_ids.shape[0] != num_requests:
+        raise KernelError("conv_tail_update: the request lists do not fit")
+    _call("lc_conv_tail_update", _ptr(proj), proj.shape[1], proj.shape[0], _ptr(tail), tail.shape[0], channels,
+          num_taps, _ptr(q_offsets), _ptr(slot_ids), num_requests, _stream())
+
+
+def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offsets: torch.Tensor,
+               slot_ids: torch.Tensor, num_requests: int, heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
+    """The delta-rule recurrence over every request's tokens in order, per head:
+    ``S <- diag(decay) S - removal (probe^T S) + write v^T`` (both terms read the old S), ``o = S^T read``.
+    ``coef`` float32 [5, T, heads key_dim] holds decay, probe, removal, write, read; ``v`` float32
+    [T, heads value_dim]; ``state`` float32 [slots, heads, key_dim, value_dim] is read at the request's
+    slot before its first token of the step and written after its last.  -> float32 [T, heads value_dim]."""
+    _need(coef, "delta_scan coef", torch.float32, 3)
+    _need(v, "delta_scan v", torch.float32, 2)
+    _need(state, "delta_scan state", torch.float32, 4)
+    T = v.shape[0]
+    if tuple(coef.shape) != (5, T, heads * key_dim) or v.shape[1] != heads * value_dim:
+        raise KernelError("delta_scan: coef or v do not fit the heads")
+    if tuple(state.shape[1:]) != (heads, key_dim, value_dim):
+        raise KernelError(f"delta_scan: state {tuple(state.shape)} does not fit [slots, {heads}, {key_dim}, {value_dim}]")
+    _need(q_offsets, "q_offsets", torch.int32, 1)
+    _need(slot_ids, "slot_ids", torch.int32, 1)
+    if q_offsets.shape[0] != num_requests + 1 or slot_ids.shape[0] != num_requests:
+        raise KernelError("delta_scan: the request lists do not fit")
+    check_delta_sizes("delta_scan", key_dim, value_dim)
+    out = torch.empty((T, heads * value_dim), dtype=torch.float32, device=v.device)
+    if T:
+        _call("lc_delta_scan", _ptr(coef), _ptr(v), _ptr(state), state.shape[0], _ptr(out), _ptr(q_offsets),
+              _ptr(slot_ids), num_requests, T, heads, key_dim, value_dim, _stream())
+    return out
+
+
+HEAD_GATES = {"sigmoid": 0, "silu": 1}
+
+
+def head_gate_norm(o: torch.Tensor, gates: torch.Tensor, gate_column: int, weight: torch.Tensor,
+                   weight_per_head: bool, eps: float, gate: str, heads: int, dim: int,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Every head of float32 ``o`` [T, heads dim] divided by its root mean square (eps inside the root),
+    times ``weight`` ([heads dim] where ``weight_per_head``, else [dim] for all heads), times
+    ``gate``(g) with g the float32 columns ``gate_column`` .. + heads dim of ``gates``.  -> [T, heads dim]."""
+    _need(o, "head_gate_norm o", torch.float32, 2)
+    _need(gates, "head_gate_norm gates", torch.float32, 2)
+    _need(weight, "head_gate_norm weight", torch.float32, 1)
+    T, n = o.shape
+    if n != heads * dim or gates.shape[0] != T or gate_column + n > gates.shape[1]:
+        raise KernelError("head_gate_norm: o or the gates do not fit the heads")
+    if weight.shape[0] != (n if weight_per_head else dim):
+        raise KernelError("head_gate_norm: the weight does not fit the heads")
+    out = torch.empty((T, n), dtype=out_dtype, device=o.device)
+    if T:
+        _call("lc_head_gate_norm", _ptr(o), _ptr(gates), gates.shape[1], gate_column, _ptr(weight),
+              1 if weight_per_head else 0, float(eps), HEAD_GATES[gate], T, heads, dim, _ptr(out), _dt(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ routing by logits, shared expert
+def moe_route_logits(logits: torch.Tensor, experts: int, top: int, bias: Optional[torch.Tensor] = None,
+                     large_tiles: bool = False) -> Routing:
+    """As :func:`moe_route`, from the first ``experts`` columns of float32 ``logits`` [T, >= experts] with
+    ``bias`` [experts] added: the ``top`` largest logits are chosen (the lower index wins a tie) and
+    weigh as the softmax over the chosen logits alone."""
+    _need(logits, "router logits", torch.float32, 2)
+    T, cols = logits.shape
+    E = experts
+    if cols < E:
+        raise KernelError(f"moe_route_logits: {cols} columns for {E} experts")
+    if bias is not None:
+        _need(bias, "router bias", torch.float32, 1)
+        if bias.shape[0] != E:
+            raise KernelError(f"moe_route_logits: a bias of {bias.shape[0]} entries for {E} experts")
+    dev = logits.device
+    ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+    weights = torch.empty((T, top), dtype=torch.float32, device=dev)
+    _call("lc_moe_route_logits", _ptr(logits), cols, _ptr(bias), T, E, top, _ptr(ids), _ptr(weights), _stream())
+    tile = 16 if T * top <= 16 * E else 128 if (large_tiles and T * top >= 192 * E) else 64
+    lists = torch.empty((2 * (E + 1) + 2 * T * top,), dtype=torch.int32, device=dev)
+    row_start, tile_start = lists[:E + 1], lists[E + 1:2 * (E + 1)]
+    sorted_token, entry_row = lists[2 * (E + 1):2 * (E + 1) + T * top], lists[2 * (E + 1) + T * top:]
+    _call("lc_moe_lists", _ptr(ids), T, top, E, tile, _ptr(row_start), _ptr(tile_start), _ptr(sorted_token),
+          _ptr(entry_row), _stream())
+    return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, tile, (T * top) // tile + E)
+
+
+def moe_combine_shared(y: torch.Tensor, routing: Routing, shared: torch.Tensor, gates: torch.Tensor,
+                       gate_column: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """:func:`moe_combine` plus ``sigmoid(gates[t, gate_column]) * shared[t]`` (``gates`` float32)."""
+    _need(y, "moe_combine_shared y", torch.float32, 2)
+    _need(shared, "moe_combine_shared shared", None, 2)
+    _need(gates, "moe_combine_shared gates", torch.float32, 2)
+    T, top = routing.ids.shape
+    n = y.shape[1]
+    if y.shape[0] != T * top or tuple(shared.shape) != (T, n) or gates.shape[0] != T or not 0 <= gate_column < gates.shape[1]:
+        raise KernelError("moe_combine_shared: the operands do not fit the routing")
+    out = torch.empty((T, n), dtype=out_dtype, device=y.device)
+    if T:
+        _call("lc_moe_combine_shared", _ptr(y), _ptr(routing.weights), _ptr(routing.entry_row), T, top, n,
+              _ptr(shared), _dt(shared), _ptr(gates), gates.shape[1], gate_column, _ptr(out), _dt(out), _stream())
+    return out

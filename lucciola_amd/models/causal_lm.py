@@ -212,7 +212,10 @@ class CausalLM:
     # ------------------------------------------------------------------ forward
     def forward(self, batch: StepBatch, sites: List[SiteView]) -> torch.Tensor:
         """Run the batch's tokens through every site; float32 logits [wanted, vocab]."""
-        stream = ResidualStream(self.embed.forward(batch.token_ids))
+        if getattr(self.embed, "takes_positions", False):
+            stream = ResidualStream(self.embed.forward(batch.token_ids, batch.positions))
+        else:
+            stream = ResidualStream(self.embed.forward(batch.token_ids))
         for index, entry in enumerate(self.spec.run_order):
             if index in self.before:
                 self.before[index].forward(stream)

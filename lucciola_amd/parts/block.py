@@ -46,3 +46,46 @@ class PreNormMixerBlock:
     def forward(self, stream: ResidualStream, site) -> None:
         x = PreNormResidualBlock._normed(self.mixer_norm, self.mixer, stream)
         stream.pending = self.mixer.forward(x, site)
+
+
+def _post_normed(norm, branch):
+    """The branch output behind its norm: left to the next kernel that adds to the stream where
+    the norm can say so (``behind``), else normed now."""
+    if hasattr(norm, "behind"):
+        return norm.behind(branch)
+    from ..kernels import ops
+    return norm.apply(ops.value(branch))
+
+
+@BLOCKS.register("sandwich_residual")
+class SandwichResidualBlock:
+    """A norm before and behind each branch: h += post(mixer(pre(h))); h += post(ff(pre(h)))."""
+
+    slots = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm",
+             "mixer_post_norm": "norm", "feed_forward_norm": "norm", "feed_forward_post_norm": "norm"}
+
+    def __init__(self, mixer, feed_forward, mixer_norm, mixer_post_norm, feed_forward_norm,
+                 feed_forward_post_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.mixer_post_norm = mixer_norm, mixer_post_norm
+        self.feed_forward_norm, self.feed_forward_post_norm = feed_forward_norm, feed_forward_post_norm
+
+    def forward(self, stream: ResidualStream, site) -> None:
+        x = self.mixer_norm.add_norm(stream)
+        stream.pending = _post_normed(self.mixer_post_norm, self.mixer.forward(x, site))
+        x = self.feed_forward_norm.add_norm(stream)
+        stream.pending = _post_normed(self.feed_forward_post_norm, self.feed_forward.forward(x))
+
+
+@BLOCKS.register("sandwich_mixer")
+class SandwichMixerBlock:
+    """The same without a feed-forward: h += post(mixer(pre(h)))."""
+
+    slots = {"mixer": "mixer", "mixer_norm": "norm", "mixer_post_norm": "norm"}
+
+    def __init__(self, mixer, mixer_norm, mixer_post_norm):
+        self.mixer, self.mixer_norm, self.mixer_post_norm = mixer, mixer_norm, mixer_post_norm
+
+    def forward(self, stream: ResidualStream, site) -> None:
+        x = self.mixer_norm.add_norm(stream)
+        stream.pending = _post_normed(self.mixer_post_norm, self.mixer.forward(x, site))

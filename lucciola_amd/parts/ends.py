@@ -47,6 +47,30 @@ class TokenEmbedding(Part):
         return ops.embedding(ids, self.weight, self.scale)
 
 
+@EMBEDDINGS.register("sinusoid_token_embedding")
+class SinusoidTokenEmbedding(TokenEmbedding):
+    """The table's row plus a position vector: entry 2i is sin(p f_i), entry 2i + 1 cos(p f_i),
+    f_i = base^(-2i/width).  The frequencies are made in float64 and kept as float32; the angle
+    and its sine and cosine are float32 arithmetic in the kernel."""
+
+    takes_positions = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, base: float = 10000.0, scale: float = 1.0):
+        super().__init__(vocab_size, hidden_size, scale)
+        self.params["base"] = base
+        self.base = float(base)
+        self.frequencies: Optional[torch.Tensor] = None
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        super().bind(tensors, ctx)
+        i = torch.arange((self.H + 1) // 2, dtype=torch.float64)
+        f = torch.pow(torch.tensor(self.base, dtype=torch.float64), -2.0 * i / self.H)
+        self.frequencies = f.to(torch.float32).to(ctx.device)
+
+    def forward(self, ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        return ops.embedding_sinusoid(ids, self.weight, positions, self.frequencies, self.scale)
+
+
 @HEADS.register("linear_head")
 class LinearHead(Part):
     graph_safe = True

@@ -1,6 +1,7 @@
 """The gated feed-forward (SwiGLU) as a part: ``down(silu(gate(x)) * up(x))``, no biases
 (reference: src/qwen.cc:762-794, src/kernels/swiglu.cu:8,31-35).  gate and up are one matrix
-product here: their weights are stacked at load."""
+product here: their weights are stacked at load.  The gate's activation is a parameter ("silu",
+or "gelu_tanh", which takes a kernel of its own behind the product)."""
 from __future__ import annotations
 
 from typing import Dict
@@ -29,9 +30,9 @@ class GatedMLP(Part):
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size,
                          activation=activation)
-        if activation != "silu":
-            raise ValueError(f"gated_mlp: activation '{activation}' has no kernel (only silu)")
-        self.H, self.I = int(hidden_size), int(intermediate_size)
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"gated_mlp: activation '{activation}' has no kernel ({', '.join(ops.GATE_ACTIVATIONS)})")
+        self.H, self.I, self.activation = int(hidden_size), int(intermediate_size), activation
 
     def declare(self) -> Dict[str, ParamDecl]:
         return {"gate_proj": ParamDecl((self.I, self.H)),
@@ -44,7 +45,7 @@ class GatedMLP(Part):
         self.dtype = ctx.dtype
         # where the matrix-core kernel takes the sizes, gate and up rows are interleaved so that
         # silu(gate) * up is formed in the product's epilogue and [T, 2 I] never reaches memory
-        self.fused = (ctx.device.type == "cuda" and self.I % 8 == 0 and gate.dtype == up.dtype
+        self.fused = (self.activation == "silu" and ctx.device.type == "cuda" and self.I % 8 == 0 and gate.dtype == up.dtype
                       and ops.gemm_swiglu_supported(ctx.dtype, gate.new_empty((2 * self.I, 1)), self.H))
         if self.fused:
             self.gate_up = ops.interleave_gate_up(gate, up)
@@ -54,8 +55,10 @@ class GatedMLP(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.fused:
             z = ops.gemm_swiglu(x, self.gate_up)
-        else:
+        elif self.activation == "silu":
             z = ops.swiglu(ops.gemm(x, self.gate_up, self.dtype))
+        else:
+            z = ops.gated_activation(ops.gemm(x, self.gate_up, self.dtype), self.activation)
         return ops.gemm(z, self.down, self.dtype, defer=True)
 
 
@@ -132,3 +135,66 @@ class RoutedMLP(Part):
         hidden = ops.moe_experts(x, self.up, routing, self.dtype, activation=self.activation, gather=True)
         y = ops.moe_experts(hidden, self.down, routing, torch.float32)
         return ops.moe_combine(y, routing, self.dtype)
+
+
+@FEED_FORWARDS.register("routed_gated_mlp")
+class RoutedGatedMLP(Part):
+    """A mixture of small gated feed-forwards ``down(act(gate x) * (up x))``.  The router's logits
+    (float32, plus a bias where ``router_bias``) pick the ``top`` largest; their weights are the
+    softmax over the chosen logits alone.  ``shared_size`` > 0: a gated feed-forward of that inner
+    size runs for every token and is added times sigmoid(w . x), one number per token (its
+    weight row rides along in the router's product).  The experts' products run over the (token,
+    choice) pairs sorted by expert, as for ``routed_mlp``; nothing passes the host."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int,
+                 activation: str = "silu", router_bias: bool = False, shared_size: int = 0):
+        super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size, experts=experts, top=top,
+                         activation=activation, router_bias=router_bias, shared_size=shared_size)
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"routed_gated_mlp: activation '{activation}' has no kernel")
+        if not 1 <= int(top) <= int(experts):
+            raise ValueError(f"routed_gated_mlp: top {top} of {experts} experts")
+        self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(experts), int(top)
+        self.activation, self.router_bias, self.S = activation, bool(router_bias), int(shared_size)
+        self.shared = (GatedMLP(hidden_size=self.H, intermediate_size=self.S, activation=activation)
+                       if self.S else None)
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        out = {"router": ParamDecl((self.E, self.H))}
+        if self.router_bias:
+            out["router_bias"] = ParamDecl((self.E,), role="vector")
+        for k in range(self.E):
+            out[f"experts.{k}.gate"] = ParamDecl((self.I, self.H))
+            out[f"experts.{k}.up"] = ParamDecl((self.I, self.H))
+            out[f"experts.{k}.down"] = ParamDecl((self.H, self.I))
+        if self.shared is not None:
+            out.update({"shared.gate": ParamDecl((self.S, self.H)), "shared.up": ParamDecl((self.S, self.H)),
+                        "shared.down": ParamDecl((self.H, self.S)), "shared_gate": ParamDecl((1, self.H))})
+        return out
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.dtype = ctx.dtype
+        # one product gives the router's logits and, in its last column, the shared expert's gate
+        self.router = stack_rows([tensors["router"]] + ([tensors["shared_gate"]] if self.shared is not None else []))
+        self.bias = tensors["router_bias"].to(torch.float32).contiguous() if self.router_bias else None
+        self.gate_up = stack_rows([t for k in range(self.E) for t in (tensors[f"experts.{k}.gate"],
+                                                                       tensors[f"experts.{k}.up"])]
+                                  ).view(self.E, 2 * self.I, self.H)
+        self.down = stack_rows([tensors[f"experts.{k}.down"] for k in range(self.E)]).view(self.E, self.H, self.I)
+        self.large_tiles = ctx.device.type == "cuda" and ops.moe_large_tiles(ctx.dtype, self.gate_up, self.down)
+        if self.shared is not None:
+            self.shared.bind({"gate_proj": tensors["shared.gate"], "up_proj": tensors["shared.up"],
+                              "down_proj": tensors["shared.down"]}, ctx)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        logits = ops.gemm(x, self.router, torch.float32)            # [T, E (+ 1)]
+        routing = ops.moe_route_logits(logits, self.E, self.top, self.bias, large_tiles=self.large_tiles)
+        both = ops.moe_experts(x, self.gate_up, routing, self.dtype, gather=True)
+        hidden = ops.gated_activation(both, self.activation)
+        y = ops.moe_experts(hidden, self.down, routing, torch.float32)
+        if self.shared is None:
+            return ops.moe_combine(y, routing, self.dtype)
+        extra = ops.value(self.shared.forward(x))
+        return ops.moe_combine_shared(y, routing, extra, logits, self.E, self.dtype)

@@ -86,3 +86,46 @@ class DynamicTanh(Part):
 
     def fused_rms(self):
         return None
+
+
+@NORMS.register("layer_norm")
+class LayerNorm(Part):
+    """``y = (x - mean) / sqrt(var + eps) * w + b`` over the last dimension, the variance being
+    the mean of the squared deviations; float32 arithmetic.  Where the branch output that waits
+    to be added is itself to be normed first (``ops.NormedBranch``: a block with a norm behind
+    each branch), one kernel norms the branch, adds it to the stream and norms the stream."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float):
+        super().__init__(size=size, eps=eps)
+        self.size, self.eps = int(size), float(eps)
+        self.weight = self.bias = None
+        self.dtype = None
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal"),
+                "bias": ParamDecl((self.size,), role="vector", init="normal")}
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        self.weight, self.bias = tensors["weight"], tensors["bias"]
+        self.dtype = ctx.dtype
+
+    def add_norm(self, stream: ResidualStream, scaled: bool = False):
+        x = ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype)
+        stream.pending = None
+        return x
+
+    def add_norm_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        return ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype, rows=rows)
+
+    def behind(self, branch) -> "ops.NormedBranch":
+        """``branch`` (a branch's output) as something that is normed by this norm before it is
+        added to the stream."""
+        return ops.NormedBranch(ops.value(branch), self.weight, self.bias, self.eps)
+
+    def apply(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layer_norm_act(x, self.weight, self.bias, self.eps)
+
+    def fused_rms(self):
+        return None

@@ -57,11 +57,22 @@ class ParamDecl:
     kernels), "int" (an integer table, kept as int32).
     init: how the random-weights mode fills it: "normal" N(0, std), "ones_plus_normal"
     1 + N(0, std) (norm weights), "zeros", "ones".
+    A size of -1 in ``shape`` is one that the checkpoint decides (an inner size that no
+    configuration key names): any size fits, the part reads it off the tensor it is given, and
+    the random-weights mode makes it ``free_size``.
     """
 
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: str = "normal"
+    free_size: int = 16
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(want in (-1, have) for want, have in zip(self.shape, shape))
+
+    def concrete_shape(self) -> Tuple[int, ...]:
+        return tuple(self.free_size if n == -1 else int(n) for n in self.shape)
 
 
 class WeightSource:
@@ -193,7 +204,7 @@ def load_declared(source: WeightSource, declared: Mapping[str, ParamDecl],
         if name not in have:
             continue
         shape, dtype = source.shape_dtype(name)
-        if tuple(shape) != tuple(decl.shape):
+        if not decl.fits(shape):
             wrong_shape.append((name, tuple(shape), tuple(decl.shape)))
         if kept_dtype(dtype, decl.role) is None:
             wrong_dtype.append((name, f"stored as {dtype}, which a {decl.role} cannot be"))

@@ -79,16 +79,17 @@ def unit_normal(key: int, first: int, count: int, device) -> torch.Tensor:
 def random_tensor(name: str, decl: ParamDecl, seed: int, std: float, dtype: torch.dtype,
                   device="cpu") -> torch.Tensor:
     dev = torch.device(device)
+    shape = decl.concrete_shape()
     if decl.role == "int":
-        return torch.zeros(decl.shape, dtype=torch.int32, device=dev)
+        return torch.zeros(shape, dtype=torch.int32, device=dev)
     if decl.init == "zeros":
-        return torch.zeros(decl.shape, dtype=dtype, device=dev)
+        return torch.zeros(shape, dtype=dtype, device=dev)
     if decl.init == "ones":
-        return torch.ones(decl.shape, dtype=dtype, device=dev)
+        return torch.ones(shape, dtype=dtype, device=dev)
     if decl.init not in ("normal", "ones_plus_normal"):
         raise ValueError(f"tensor '{name}': unknown init '{decl.init}'")
     count = 1
-    for n in decl.shape:
+    for n in shape:
         count *= int(n)
     key = tensor_key(seed, name)
     out = torch.empty(count, dtype=dtype, device=dev)
@@ -99,7 +100,7 @@ def random_tensor(name: str, decl: ParamDecl, seed: int, std: float, dtype: torc
         if decl.init == "ones_plus_normal":
             t = t + 1.0
         out[first:first + n] = t.to(dtype)
-    return out.view(tuple(decl.shape))
+    return out.view(shape)
 
 
 def random_tensors(declared: Mapping[str, ParamDecl], seed: int, std: float,

@@ -75,7 +75,7 @@ def attention(qkv, batch, k_cache, v_cache, nh, nkv, d, page_size, scale, window
                            batch.positions, prologue.rope_table, k_cache, v_cache, prologue.slots,
                            page_size)
     T = qkv.shape[0]
-    q = qkv.view(T, nh + 2 * nkv, d)[:, :nh].to(F64)
+    q = qkv[:, :nh * d].reshape(T, nh, d).to(F64)     # the q heads come first (alone, or with k and v behind)
     out = torch.zeros(T, nh, d, dtype=F64, device=qkv.device)
     group = nh // nkv
     tok_req = batch.tok_req.tolist()
@@ -268,7 +268,198 @@ def feed_tokens(ids, source, sampled):
     ids[take] = sampled[source[take].long()]
 
 
-ALL = ("feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
+# ------------------------------------------------------------------ layer norm, position vector, heads in slots
+def _layer_norm64(v, weight, bias, eps):
+    mean = v.mean(-1, keepdim=True)
+    dev = v - mean
+    return dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + eps) * weight.to(F64) + bias.to(F64)
+
+
+def layer_norm_act(x, weight, bias, eps):
+    return _layer_norm64(x.to(F64), weight, bias, eps).to(x.dtype)
+
+
+def layer_norm(h, delta, weight, bias, eps, out_dtype, rows=None):
+    from lucciola_amd.kernels import ops
+    if isinstance(delta, ops.NormedBranch):
+        delta = _layer_norm64(delta.x.to(F64), delta.weight, delta.bias, delta.eps).to(torch.float32)
+    elif delta is not None and not isinstance(delta, torch.Tensor):
+        delta = delta.value()
+    if rows is None:
+        if delta is not None:
+            h += delta.to(torch.float32)
+        v = h.to(F64)
+    else:
+        v = h[rows.long()].to(F64)
+        if delta is not None:
+            v = (h[rows.long()] + delta[rows.long()].to(torch.float32)).to(F64)
+    return _layer_norm64(v, weight, bias, eps).to(out_dtype)
+
+
+def embedding_sinusoid(ids, table, positions, frequencies, scale=1.0):
+    H = table.shape[1]
+    angle = positions.to(torch.float32)[:, None] * frequencies[None, :]
+    out = table[ids.long()].to(torch.float32) * scale
+    out[:, 0::2] += torch.sin(angle)
+    out[:, 1::2] += torch.cos(angle)[:, :H // 2]
+    return out
+
+
+def gated_activation(gu, kind):
+    I = gu.shape[1] // 2
+    g, u = gu[:, :I].to(F64), gu[:, I:].to(F64)
+    a = g / (1 + torch.exp(-g)) if kind == "silu" else _act(g, kind)
+    return (a * u).to(gu.dtype)
+
+
+def attention_head_slot(size):
+    for slot in (32, 64, 96, 128):
+        if size <= slot:
+            return slot
+    return -(-size // 16) * 16
+
+
+def head_norm_write(proj, nh, nkv, d, dv, slot, q_weight, k_weight, eps, head_scale, k_cache, v_cache, slots,
+                    page_size):
+    T = proj.shape[0]
+    q = proj[:, :nh * d].view(T, nh, d).to(F64)
+    if q_weight is not None:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.to(F64)
+    if head_scale is not None:
+        q = q * head_scale.to(F64)[None, :, None]
+    out = torch.zeros(T, nh, slot, dtype=proj.dtype, device=proj.device)
+    out[:, :, :d] = q.to(proj.dtype)
+    if nkv and slots is not None and k_cache is not None:
+        k = proj[:, nh * d: (nh + nkv) * d].view(T, nkv, d).to(F64)
+        if k_weight is not None:
+            k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.to(F64)
+        v = proj[:, (nh + nkv) * d:].view(T, nkv, dv)
+        for t in range(T):
+            s = int(slots[t])
+            if s < 0:
+                continue
+            page, off = divmod(s, page_size)
+            k_cache[page, :, off, :] = 0
+            k_cache[page, :, off, :d] = k[t].to(k_cache.dtype)
+            v_cache[page, :, :, off] = 0
+            v_cache[page, :, :dv, off] = v[t].to(v_cache.dtype)
+    return out.view(T, nh * slot)
+
+
+# ------------------------------------------------------------------ delta rules
+def check_delta_sizes(what, key_dim, value_dim, taps=1):
+    pass
+
+
+def general_delta_prepare(proj, heads, dim, inner, decay_out, decay_bias, removal_bias, unit_eps, decay_scale):
+    T, n = proj.shape[0], heads * dim
+    p = proj.to(F64)
+    r, k, v, removal, decay_in = p[:, :n], p[:, n:2 * n], p[:, 2 * n:3 * n], p[:, 4 * n:5 * n], p[:, 5 * n:]
+    w = torch.exp(-decay_scale * torch.sigmoid(torch.tanh(decay_in) @ decay_out.to(F64).T + decay_bias.to(F64)))
+    a = torch.sigmoid(removal + removal_bias.to(F64))
+    kh = k.view(T, heads, dim)
+    u = (kh / torch.sqrt((kh * kh).sum(-1, keepdim=True) + unit_eps)).view(T, n)
+    coef = torch.stack([w, u, a * u, k, r]).to(torch.float32)
+    return coef, v.to(torch.float32).contiguous()
+
+
+def _conv_inputs(proj, tail, C, K, tok_req, q_offsets, slot_ids):
+    """[K, T, C]: input j steps back of every token and channel."""
+    T = proj.shape[0]
+    x = torch.zeros(K, T, C, dtype=F64)
+    starts = q_offsets.tolist()
+    for t in range(T):
+        r = int(tok_req[t])
+        n = t - starts[r]
+        for j in range(K):
+            if j <= n:
+                x[j, t] = proj[t - j, :C].to(F64)
+            else:
+                x[j, t] = tail[int(slot_ids[r]), (K - 1) - (j - n)].to(F64)
+    return x
+
+
+def gated_delta_prepare(proj, tail, taps, rate_log, rate_bias, heads, kv_heads, key_dim, value_dim, num_taps,
+                        unit_eps, tok_req, q_offsets, slot_ids):
+    T = proj.shape[0]
+    nk, nv = kv_heads * key_dim, heads * value_dim
+    C = 2 * nk + nv
+    x = _conv_inputs(proj, tail, C, num_taps, tok_req, q_offsets, slot_ids)
+    y = torch.zeros(T, C, dtype=F64)
+    for j in range(num_taps):
+        y += x[j] * taps.to(F64)[:, num_taps - 1 - j][None, :]
+    y = y / (1 + torch.exp(-y))
+    q, k, v = y[:, :nk].view(T, kv_heads, key_dim), y[:, nk:2 * nk].view(T, kv_heads, key_dim), y[:, 2 * nk:]
+    q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * key_dim ** -0.5
+    k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+    rep = heads // kv_heads
+    q, k = q.repeat_interleave(rep, dim=1), k.repeat_interleave(rep, dim=1)        # [T, heads, key_dim]
+    beta = torch.sigmoid(proj[:, C + nv: C + nv + heads].to(F64))[:, :, None]
+    rate = proj[:, C + nv + heads:].to(F64) + rate_bias.to(F64)
+    g = torch.exp(-torch.exp(rate_log.to(F64)) * torch.nn.functional.softplus(rate))[:, :, None]
+    coef = torch.stack([g.expand_as(k), g * k, beta * k, beta * k, q]).reshape(5, T, heads * key_dim)
+    return coef.to(torch.float32).contiguous(), v.to(torch.float32).contiguous()
+
+
+def conv_tail_update(proj, tail, channels, num_taps, q_offsets, slot_ids, num_requests):
+    if num_taps <= 1:
+        return
+    starts = q_offsets.tolist()
+    for r in range(num_requests):
+        s = int(slot_ids[r])
+        rows = torch.cat([tail[s], proj[starts[r]:starts[r + 1], :channels].to(tail.dtype)], dim=0)
+        tail[s] = rows[-(num_taps - 1):]
+
+
+def delta_scan(coef, v, state, q_offsets, slot_ids, num_requests, heads, key_dim, value_dim):
+    T = v.shape[0]
+    c = coef.to(F64).view(5, T, heads, key_dim)
+    vv = v.to(F64).view(T, heads, value_dim)
+    out = torch.zeros(T, heads, value_dim, dtype=F64)
+    starts = q_offsets.tolist()
+    for r in range(num_requests):
+        S = state[int(slot_ids[r])].to(F64)                    # [heads, key, value]
+        for t in range(starts[r], starts[r + 1]):
+            taken = torch.einsum("hk,hkv->hv", c[1, t], S)
+            S = c[0, t][:, :, None] * S - c[2, t][:, :, None] * taken[:, None, :] + c[3, t][:, :, None] * vv[t][:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, c[4, t])
+        state[int(slot_ids[r])] = S.to(state.dtype)
+    return out.view(T, heads * value_dim).to(torch.float32)
+
+
+def head_gate_norm(o, gates, gate_column, weight, weight_per_head, eps, gate, heads, dim, out_dtype):
+    T = o.shape[0]
+    x = o.to(F64).view(T, heads, dim)
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    w = weight.to(F64).view(heads, dim) if weight_per_head else weight.to(F64)[None, :]
+    g = gates[:, gate_column:gate_column + heads * dim].to(F64).view(T, heads, dim)
+    g = torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g)
+    return (x * w * g).view(T, heads * dim).to(out_dtype)
+
+
+def moe_route_logits(logits, experts, top, bias=None, large_tiles=False):
+    z = logits[:, :experts].to(F64)
+    if bias is not None:
+        z = z + bias.to(F64)
+    picked, ids = torch.topk(z, top, dim=-1)
+    r = _Routing()
+    r.ids, r.weights = ids.to(torch.int32), torch.softmax(picked, dim=-1).to(torch.float32)
+    return r
+
+
+def moe_combine_shared(y, routing, shared, gates, gate_column, out_dtype):
+    T, top = routing.ids.shape
+    total = (y.to(F64).view(T, top, -1) * routing.weights.to(F64)[:, :, None]).sum(1)
+    return (total + torch.sigmoid(gates[:, gate_column].to(F64))[:, None] * shared.to(F64)).to(out_dtype)
+
+
+def moe_large_tiles(x_dtype, up, down):
+    return False
+
+
+ALL = ("layer_norm", "layer_norm_act", "embedding_sinusoid", "gated_activation", "attention_head_slot", "head_norm_write",
+       "check_delta_sizes", "general_delta_prepare", "gated_delta_prepare", "conv_tail_update", "delta_scan",
+       "head_gate_norm", "moe_route_logits", "moe_combine_shared", "feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample", "dynamic_tanh", "stream_add", "activation", "gemm_act", "grouped_gemm",
        "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine")
 
