@@ -1,0 +1,297 @@
+// Mixers that keep a matrix of state per head and request: the delta-rule recurrence and what
+// turns a layer's projections into its inputs.  Everything here is float32.
+//
+// The recurrence, per head, with the state S [key, value] and per token the vectors decay,
+// probe, removal, write, read over the key channels and the value v:
+//     S <- diag(decay) S - removal (probe^T S) + write v^T        (both terms read the old S)
+//     o  = S^T read
+// A column of S (one value channel) never meets another, so the work is shared out by columns:
+// a workgroup owns 16 columns of one head of one request and walks the request's tokens in
+// order; a column belongs to 16 neighbouring lanes, lane l holding the key rows l, l + 16, ...
+// in registers.  The tokens' vectors come through LDS a chunk of tokens at a time.
+//
+// The two delta rules differ in how the five vectors are made:
+//   generalized   decay = exp(-c sigmoid(W2 tanh(x1) + w0)), a = sigmoid(xa + ba), u = k / sqrt(|k|^2 + e):
+//                 probe = u, removal = a u, write = k, read = r
+//   gated         q, k, v through a short causal convolution per channel and silu; q, k unit vectors,
+//                 q times key_dim^-1/2; g = exp(-exp(A) softplus(xg + bg)), beta = sigmoid(xb):
+//                 decay = g, probe = g k, removal = beta k, write = beta k, read = q
+#include "common.h"
+
+#include "activations.h"
+
+namespace lc {
+
+constexpr int DELTA_MAX_KEY = 256;
+constexpr int DELTA_PER_LANE = DELTA_MAX_KEY / kWave;
+constexpr int DELTA_MAX_INNER = 1024;
+constexpr int CONV_MAX_TAPS = 16;
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// One wave per (token, head).  proj [T, 5 n + inner]: r | k | v | gate | removal | decay_in.
+__global__ __launch_bounds__(kWave) void general_delta_prepare_kernel(
+    const float* __restrict__ proj, int T, int heads, int dim, int inner, const float* __restrict__ decay_out,
+    const float* __restrict__ decay_bias, const float* __restrict__ removal_bias, float unit_eps, float decay_scale,
+    float* __restrict__ coef, float* __restrict__ v_out) {
+    __shared__ float hidden[DELTA_MAX_INNER];
+    const int t = blockIdx.x / heads, head = blockIdx.x % heads, lane = threadIdx.x;
+    const int n = heads * dim;
+    const size_t cols = (size_t)5 * n + inner;
+    const float* row = proj + (size_t)t * cols;
+    for (int j = lane; j < inner; j += kWave) hidden[j] = tanhf(row[(size_t)5 * n + j]);
+    __syncthreads();
+    float k[DELTA_PER_LANE], ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < DELTA_PER_LANE; ++e) {
+        const int i = lane + kWave * e;
+        k[e] = i < dim ? row[n + head * dim + i] : 0.f;
+        ss = fmaf(k[e], k[e], ss);
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) + unit_eps);
+    const size_t plane = (size_t)T * n;
+#pragma unroll
+    for (int e = 0; e < DELTA_PER_LANE; ++e) {
+        const int i = lane + kWave * e;
+        if (i >= dim) continue;
+        const int c = head * dim + i;
+        float z = decay_bias[c];
+        const float* w2 = decay_out + (size_t)c * inner;
+        for (int j = 0; j < inner; ++j) z = fmaf(hidden[j], w2[j], z);
+        const float decay = expf(-decay_scale * sigmoid(z));
+        const float a = sigmoid(row[(size_t)4 * n + c] + removal_bias[c]);
+        const float u = k[e] * inv;
+        const size_t at = (size_t)t * n + c;
+        coef[at] = decay;
+        coef[plane + at] = u;
+        coef[2 * plane + at] = a * u;
+        coef[3 * plane + at] = k[e];
+        coef[4 * plane + at] = row[c];
+        v_out[at] = row[(size_t)2 * n + c];
+    }
+}
+
+// Channel c of token t through the convolution: sum_j taps[c, K - 1 - j] x[t - j, c], where an input
+// from before the step comes from the request's tail (its last K - 1 inputs, oldest first).
+__device__ __forceinline__ float conv_at(const float* __restrict__ proj, size_t cols, int t, int local, int c,
+                                         const float* __restrict__ taps, int K, const float* __restrict__ tail, int C) {
+    float y = 0.f;
+    for (int j = 0; j < K; ++j) {
+        const float x = j <= local ? proj[(size_t)(t - j) * cols + c]
+                                   : tail[(size_t)((K - 1) - (j - local)) * C + c];
+        y = fmaf(taps[(size_t)c * K + (K - 1 - j)], x, y);
+    }
+    return y;
+}
+
+// One wave per (token, head).  proj [T, C + nv + 2 heads]: q | k | v | gate | beta | rate.
+__global__ __launch_bounds__(kWave) void gated_delta_prepare_kernel(
+    const float* __restrict__ proj, int T, int heads, int kv_heads, int dk, int dv, int K,
+    const float* __restrict__ taps, const float* __restrict__ tails, const float* __restrict__ rate_log,
+    const float* __restrict__ rate_bias, float unit_eps, const int* __restrict__ tok_req,
+    const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, float* __restrict__ coef,
+    float* __restrict__ v_out) {
+    const int t = blockIdx.x / heads, head = blockIdx.x % heads, lane = threadIdx.x;
+    const int nk = kv_heads * dk, nv = heads * dv, C = 2 * nk + nv;
+    const size_t cols = (size_t)C + nv + 2 * heads;
+    const int r = tok_req[t];
+    const int local = t - q_offsets[r];
+    const float* tail = tails + (size_t)slot_ids[r] * (K - 1) * C;
+    const int kv = head / (heads / kv_heads);
+    float q[DELTA_PER_LANE], k[DELTA_PER_LANE], qq = 0.f, kk = 0.f;
+#pragma unroll
+    for (int e = 0; e < DELTA_PER_LANE; ++e) {
+        const int i = lane + kWave * e;
+        q[e] = k[e] = 0.f;
+        if (i < dk) {
+            q[e] = silu_f(conv_at(proj, cols, t, local, kv * dk + i, taps, K, tail, C));
+            k[e] = silu_f(conv_at(proj, cols, t, local, nk + kv * dk + i, taps, K, tail, C));
+        }
+        qq = fmaf(q[e], q[e], qq);
+        kk = fmaf(k[e], k[e], kk);
+    }
+    const float q_inv = 1.f / (sqrtf(wave_sum(qq) + unit_eps) * sqrtf((float)dk));
+    const float k_inv = 1.f / sqrtf(wave_sum(kk) + unit_eps);
+    const float* row = proj + (size_t)t * cols;
+    const float beta = sigmoid(row[(size_t)C + nv + head]);
+    const float g = expf(-expf(rate_log[head]) * softplus_f(row[(size_t)C + nv + heads + head] + rate_bias[head]));
+    const size_t plane = (size_t)T * heads * dk;
+#pragma unroll
+    for (int e = 0; e < DELTA_PER_LANE; ++e) {
+        const int i = lane + kWave * e;
+        if (i >= dk) continue;
+        const size_t at = ((size_t)t * heads + head) * dk + i;
+        const float key = k[e] * k_inv;
+        coef[at] = g;
+        coef[plane + at] = g * key;
+        coef[2 * plane + at] = beta * key;
+        coef[3 * plane + at] = beta * key;
+        coef[4 * plane + at] = q[e] * q_inv;
+    }
+    for (int i = lane; i < dv; i += kWave)
+        v_out[((size_t)t * heads + head) * dv + i] =
+            silu_f(conv_at(proj, cols, t, local, 2 * nk + head * dv + i, taps, K, tail, C));
+}
+
+// A thread per (request, channel): the new tail is the last K - 1 of (old tail, the step's inputs).
+__global__ void conv_tail_update_kernel(const float* __restrict__ proj, int cols, float* __restrict__ tails, int C,
+                                        int K, const int* __restrict__ q_offsets, const int* __restrict__ slot_ids) {
+    const int r = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int first = q_offsets[r], n = q_offsets[r + 1] - first;
+    float* tail = tails + (size_t)slot_ids[r] * (K - 1) * C;
+    float keep[CONV_MAX_TAPS];
+    for (int m = 0; m < K - 1; ++m) {
+        const int at = n + m;               // place in (old tail, inputs)
+        keep[m] = at < K - 1 ? tail[(size_t)at * C + c] : proj[(size_t)(first + at - (K - 1)) * cols + c];
+    }
+    for (int m = 0; m < K - 1; ++m) tail[(size_t)m * C + c] = keep[m];
+}
+
+constexpr int SCAN_COLUMNS = 16;      // value channels of a workgroup
+constexpr int SCAN_LANES = 16;        // lanes that share a column's key rows
+constexpr int SCAN_THREADS = SCAN_COLUMNS * SCAN_LANES;
+
+__device__ __forceinline__ float lanes16_sum(float v) {
+    v += __shfl_xor(v, 1, kWave);
+    v += __shfl_xor(v, 2, kWave);
+    v += __shfl_xor(v, 4, kWave);
+    v += __shfl_xor(v, 8, kWave);
+    return v;
+}
+
+// grid (column blocks, heads, requests).  ROWS key rows a lane (16 ROWS >= dk), CHUNK tokens a stage.
+template <int ROWS, int CHUNK>
+__global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
+    const float* __restrict__ coef, const float* __restrict__ v, float* __restrict__ state, float* __restrict__ out,
+    const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, int T, int heads, int dk, int dv) {
+    constexpr int DKP = ROWS * SCAN_LANES;                 // key rows with padding
+    __shared__ float vec[5][CHUNK][DKP];
+    __shared__ float val[CHUNK][SCAN_COLUMNS];
+    const int tid = threadIdx.x;
+    const int col = tid / SCAN_LANES, lane = tid % SCAN_LANES;
+    const int head = blockIdx.y, req = blockIdx.z;
+    const int j = blockIdx.x * SCAN_COLUMNS + col;         // the value channel
+    const int first = q_offsets[req], last = q_offsets[req + 1];
+    float* S_home = state + ((size_t)slot_ids[req] * heads + head) * dk * dv;
+    float S[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int i = lane + SCAN_LANES * r;
+        S[r] = (i < dk && j < dv) ? S_home[(size_t)i * dv + j] : 0.f;
+    }
+    const size_t plane = (size_t)T * heads * dk;
+    for (int t0 = first; t0 < last; t0 += CHUNK) {
+        const int count = min(CHUNK, last - t0);
+        __syncthreads();                                   // the stage before has been read
+        for (int idx = tid; idx < 5 * CHUNK * DKP; idx += SCAN_THREADS) {
+            const int i = idx % DKP, tt = (idx / DKP) % CHUNK, c = idx / (DKP * CHUNK);
+            vec[c][tt][i] = (tt < count && i < dk) ? coef[c * plane + ((size_t)(t0 + tt) * heads + head) * dk + i] : 0.f;
+        }
+        for (int idx = tid; idx < CHUNK * SCAN_COLUMNS; idx += SCAN_THREADS) {
+            const int cc = idx % SCAN_COLUMNS, tt = idx / SCAN_COLUMNS;
+            const int jj = blockIdx.x * SCAN_COLUMNS + cc;
+            val[tt][cc] = (tt < count && jj < dv) ? v[((size_t)(t0 + tt) * heads + head) * dv + jj] : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < count; ++tt) {
+            float taken = 0.f;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) taken = fmaf(vec[1][tt][lane + SCAN_LANES * r], S[r], taken);
+            taken = lanes16_sum(taken);
+            const float value = val[tt][col];
+            float read = 0.f;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const int i = lane + SCAN_LANES * r;
+                float s = vec[0][tt][i] * S[r];
+                s = fmaf(-vec[2][tt][i], taken, s);
+                s = fmaf(vec[3][tt][i], value, s);
+                S[r] = s;
+                read = fmaf(s, vec[4][tt][i], read);
+            }
+            read = lanes16_sum(read);
+            if (lane == 0 && j < dv) out[((size_t)(t0 + tt) * heads + head) * dv + j] = read;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int i = lane + SCAN_LANES * r;
+        if (i < dk && j < dv) S_home[(size_t)i * dv + j] = S[r];
+    }
+}
+
+}  // namespace lc
+
+using namespace lc;
+
+LC_API int lc_general_delta_prepare(const float* proj, int T, int heads, int dim, int inner, const float* decay_out,
+                                    const float* decay_bias, const float* removal_bias, float unit_eps,
+                                    float decay_scale, float* coef, float* v_out, hipStream_t stream) {
+    LC_CHECK(T >= 0 && heads > 0 && dim > 0 && inner >= 0, "general_delta_prepare: bad sizes");
+    LC_CHECK(dim <= DELTA_MAX_KEY, "general_delta_prepare: heads of %d key channels are above %d", dim, DELTA_MAX_KEY);
+    LC_CHECK(inner <= DELTA_MAX_INNER, "general_delta_prepare: an inner size of %d is above %d", inner, DELTA_MAX_INNER);
+    if (T == 0) return 0;
+    LC_CHECK(proj && decay_bias && removal_bias && coef && v_out && (decay_out || inner == 0),
+             "general_delta_prepare: null pointer");
+    LC_CHECK((long long)T * heads < (1ll << 31), "general_delta_prepare: too many heads");
+    general_delta_prepare_kernel<<<T * heads, kWave, 0, stream>>>(proj, T, heads, dim, inner, decay_out, decay_bias,
+                                                                  removal_bias, unit_eps, decay_scale, coef, v_out);
+    LC_LAUNCH_CHECK("general_delta_prepare");
+    return 0;
+}
+
+LC_API int lc_gated_delta_prepare(const float* proj, int T, int heads, int kv_heads, int dk, int dv, int K,
+                                  const float* taps, const float* tails, int tail_slots, const float* rate_log,
+                                  const float* rate_bias, float unit_eps, const int* tok_req, const int* q_offsets,
+                                  const int* slot_ids, float* coef, float* v_out, hipStream_t stream) {
+    LC_CHECK(T >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dk > 0 && dv > 0,
+             "gated_delta_prepare: bad sizes");
+    LC_CHECK(dk <= DELTA_MAX_KEY, "gated_delta_prepare: heads of %d key channels are above %d", dk, DELTA_MAX_KEY);
+    LC_CHECK(K >= 1 && K <= CONV_MAX_TAPS, "gated_delta_prepare: %d taps are outside 1..%d", K, CONV_MAX_TAPS);
+    if (T == 0) return 0;
+    LC_CHECK(proj && taps && rate_log && rate_bias && tok_req && q_offsets && slot_ids && coef && v_out &&
+                 (tails || K == 1) && tail_slots >= 0,
+             "gated_delta_prepare: null pointer");
+    LC_CHECK((long long)T * heads < (1ll << 31), "gated_delta_prepare: too many heads");
+    gated_delta_prepare_kernel<<<T * heads, kWave, 0, stream>>>(proj, T, heads, kv_heads, dk, dv, K, taps, tails,
+                                                                rate_log, rate_bias, unit_eps, tok_req, q_offsets,
+                                                                slot_ids, coef, v_out);
+    LC_LAUNCH_CHECK("gated_delta_prepare");
+    return 0;
+}
+
+LC_API int lc_conv_tail_update(const float* proj, int cols, int T, float* tails, int tail_slots, int C, int K,
+                               const int* q_offsets, const int* slot_ids, int R, hipStream_t stream) {
+    LC_CHECK(T >= 0 && C > 0 && cols >= C && K >= 1 && K <= CONV_MAX_TAPS && R >= 0 && tail_slots >= 0,
+             "conv_tail_update: bad sizes");
+    if (R == 0 || K == 1) return 0;
+    LC_CHECK(proj && tails && q_offsets && slot_ids, "conv_tail_update: null pointer");
+    LC_CHECK(R <= 65535, "conv_tail_update: %d requests are above the grid's 65535", R);
+    conv_tail_update_kernel<<<dim3((C + 255) / 256, R), 256, 0, stream>>>(proj, cols, tails, C, K, q_offsets, slot_ids);
+    LC_LAUNCH_CHECK("conv_tail_update");
+    return 0;
+}
+
+LC_API int lc_delta_scan(const float* coef, const float* v, float* state, int slots, float* out, const int* q_offsets,
+                         const int* slot_ids, int R, int T, int heads, int dk, int dv, hipStream_t stream) {
+    LC_CHECK(R >= 0 && T >= 0 && heads > 0 && dk > 0 && dv > 0 && slots >= 0, "delta_scan: bad sizes");
+    LC_CHECK(dk <= DELTA_MAX_KEY, "delta_scan: heads of %d key channels are above %d", dk, DELTA_MAX_KEY);
+    if (R == 0 || T == 0) return 0;
+    LC_CHECK(coef && v && state && out && q_offsets && slot_ids, "delta_scan: null pointer");
+    LC_CHECK(R <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for the grid");
+    const dim3 grid((dv + SCAN_COLUMNS - 1) / SCAN_COLUMNS, heads, R);
+#define LC_SCAN(ROWS, CHUNK)                                                                                      \
+    delta_scan_kernel<ROWS, CHUNK><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets, slot_ids, T, \
+                                                                      heads, dk, dv)
+    if (dk <= 16) LC_SCAN(1, 16);
+    else if (dk <= 32) LC_SCAN(2, 16);
+    else if (dk <= 64) LC_SCAN(4, 16);
+    else if (dk <= 128) LC_SCAN(8, 16);
+    else LC_SCAN(16, 8);
+#undef LC_SCAN
+    LC_LAUNCH_CHECK("delta_scan");
+    return 0;
+}

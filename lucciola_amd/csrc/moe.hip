@@ -66,6 +66,44 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
     if (lane < top) weights[(size_t)t * top + lane] = mine / div;
 }
 
+// One wave per token: the `top` largest of logits + bias (the lower index wins a tie), weighing as
+// the softmax over the chosen logits alone.  `cols`: entries of a row of `logits` (>= E).
+__global__ __launch_bounds__(kWave) void moe_route_logits_kernel(const float* __restrict__ logits, int cols,
+                                                                const float* __restrict__ bias, int E, int top,
+                                                                int* __restrict__ ids, float* __restrict__ weights) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (size_t)t * cols;
+    float s[MOE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i) {
+        const int e = lane + kWave * i;
+        s[i] = e < E ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    }
+    float first = 0.f, picked_sum = 0.f, mine = 0.f;      // lane k keeps exp(k-th chosen logit - the largest)
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (s[i] > best) { best = s[i]; at = lane + kWave * i; }     // a lane's experts in rising order
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, kWave);
+            const int oa = __shfl_xor(at, off, kWave);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (lane + kWave * i == at) s[i] = -INFINITY;
+        if (k == 0) first = best;
+        const float w = expf(best - first);
+        if (lane == 0) ids[(size_t)t * top + k] = at < E ? at : 0;
+        if (lane == k) mine = w;
+        picked_sum += w;
+    }
+    if (lane < top) weights[(size_t)t * top + lane] = mine / picked_sum;
+}
+
 // One workgroup: counts, the two running sums, and every pair's sorted row.
 __global__ __launch_bounds__(1024) void moe_lists_kernel(const int* __restrict__ ids, int n, int top, int E,
                                                          int tile, int* __restrict__ row_start,
@@ -108,6 +146,22 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __r
         for (int k = 0; k < top; ++k)
             total = fmaf(weights[(size_t)t * top + k], y[(size_t)entry_row[(size_t)t * top + k] * n + i], total);
         out[(size_t)t * n + i] = from_f32<T>(total);
+    }
+}
+
+// the same plus sigmoid(gates[t, gate_column]) * shared[t]
+template <typename T, typename TS>
+__global__ void moe_combine_shared_kernel(const float* __restrict__ y, const float* __restrict__ weights,
+                                          const int* __restrict__ entry_row, int top, int n,
+                                          const TS* __restrict__ shared, const float* __restrict__ gates, int gate_cols,
+                                          int gate_column, T* __restrict__ out) {
+    const int t = blockIdx.x;
+    const float g = 1.f / (1.f + expf(-gates[(size_t)t * gate_cols + gate_column]));
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float total = 0.f;
+        for (int k = 0; k < top; ++k)
+            total = fmaf(weights[(size_t)t * top + k], y[(size_t)entry_row[(size_t)t * top + k] * n + i], total);
+        out[(size_t)t * n + i] = from_f32<T>(fmaf(g, to_f32(shared[(size_t)t * n + i]), total));
     }
 }
 
@@ -155,5 +209,41 @@ LC_API int lc_moe_combine(const float* y, const float* weights, const int* entry
     else
         LC_CHECK(false, "moe combine: unknown dtype %d", dt);
     LC_LAUNCH_CHECK("moe_combine");
+    return 0;
+}
+
+// logits float32 [T, cols] (the experts' in the first E columns), bias [E] or null -> ids, weights [T, top]
+LC_API int lc_moe_route_logits(const float* logits, int cols, const float* bias, int T, int E, int top, int* ids,
+                               float* weights, hipStream_t stream) {
+    LC_CHECK(T >= 0 && E > 0 && top > 0 && top <= E && cols >= E, "moe route: bad sizes T=%d E=%d top=%d cols=%d", T, E,
+             top, cols);
+    LC_CHECK(E <= MOE_MAX_EXPERTS, "moe route: %d experts are above the supported %d", E, MOE_MAX_EXPERTS);
+    LC_CHECK(top <= kWave, "moe route: %d choices a token are above the supported %d", top, kWave);
+    if (T == 0) return 0;
+    LC_CHECK(logits && ids && weights, "moe route: null pointer");
+    moe_route_logits_kernel<<<T, kWave, 0, stream>>>(logits, cols, bias, E, top, ids, weights);
+    LC_LAUNCH_CHECK("moe_route_logits");
+    return 0;
+}
+
+// y float32 [T * top, n], shared [T, n], gates float32 [T, gate_cols] -> out [T, n]
+LC_API int lc_moe_combine_shared(const float* y, const float* weights, const int* entry_row, int T, int top, int n,
+                                 const void* shared, int dt_shared, const float* gates, int gate_cols, int gate_column,
+                                 void* out, int dt, hipStream_t stream) {
+    LC_CHECK(T >= 0 && top > 0 && n > 0 && gate_cols > 0 && gate_column >= 0 && gate_column < gate_cols,
+             "moe combine: bad sizes");
+    if (T == 0) return 0;
+    LC_CHECK(y && weights && entry_row && shared && gates && out, "moe combine: null pointer");
+    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+#define LC_COMBINE(TO, TS)                                                                                       \
+    moe_combine_shared_kernel<TO, TS><<<T, threads, 0, stream>>>(y, weights, entry_row, top, n, (const TS*)shared, \
+                                                                 gates, gate_cols, gate_column, (TO*)out)
+    if (dt == DT_F32 && dt_shared == DT_F32) LC_COMBINE(float, float);
+    else if (dt == DT_F32 && dt_shared == DT_BF16) LC_COMBINE(float, bf16);
+    else if (dt == DT_BF16 && dt_shared == DT_F32) LC_COMBINE(bf16, float);
+    else if (dt == DT_BF16 && dt_shared == DT_BF16) LC_COMBINE(bf16, bf16);
+    else LC_CHECK(false, "moe combine: unknown dtypes %d, %d", dt, dt_shared);
+#undef LC_COMBINE
+    LC_LAUNCH_CHECK("moe_combine_shared");
     return 0;
 }

@@ -240,3 +240,14 @@ def forward(cfg, weights, ids, streams=None):
         if streams is not None:
             streams.append(x.clone())
     return linear(norm_of(weights, "final.norm", x, eps), weights["head"])
+
+
+def greedy(cfg, weights, prompt, new_tokens):
+    """Greedy generation by running the whole sequence again for every token; ties go to the
+    lowest index."""
+    ids, out = list(prompt), []
+    for _ in range(new_tokens):
+        tok = int(torch.argmax(forward(cfg, weights, ids)[-1]))
+        out.append(tok)
+        ids.append(tok)
+    return out

@@ -1,0 +1,596 @@
+"""The Larupel design on the GPU: every kernel it brought against the plain torch version of the
+same operation, and the engine against the plain whole-sequence implementation
+(``plain_larupel``) in the four families of traces, in float32 and in bfloat16."""
+import pytest
+import torch
+
+import larupel_configs as lc
+import plain_larupel
+import reference_ops
+import traces
+from helpers import compare, make_runner, prompts_for, random_weights, replay
+from lucciola_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# A row's error: root mean square of the difference of the logits, means taken off, over that of the
+# plain logits.  Rounding grows along the recurrences and where a norm meets a small variance, so in
+# float32 a few rows of a hundred may go over the bound, none over three times it.  In bfloat16 the
+# roundings of the activations between the kernels alone (the plain torch versions of the kernels
+# in float64, rounding where the engine rounds) put the median row of these narrow, deep models at
+# 2 % and one row in fourteen over 10 %, and a router's choice between two experts whose logits
+# nearly tie can fall the other way, which changes that row by any amount: the bound is on the
+# median row, on the share of rows over 10 % and on the share of rows that are unrelated.  What a
+# fault of the cache, the state or the batch does wrong shows in many rows, and in float32.
+TOL = {"float32": 4e-5, "bfloat16": 1e-1}
+LENGTHS = {"A": [5, 1, 47, 90, 130], "B": [2, 61, 33, 100], "C": [150, 9, 230, 70]}
+_cache = {}
+
+
+def case(key):
+    if key not in _cache:
+        cfg, page, seed = lc.ALL[key]
+        weights = weights_for(cfg, seed, lc.STD)
+        prompts = prompts_for({"vocab_size": cfg["vocab"]}, LENGTHS[key], seed)
+        refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+        _cache[key] = (cfg, page, weights, prompts, refs)
+    return _cache[key]
+
+
+def check_rows(got, prompts, refs, dtype, every=True):
+    errors = []
+    for name, ids in prompts.items():
+        for pos in range(len(ids)):
+            if (name, pos) not in got:
+                assert not every, f"{name} position {pos}: no logits"
+                continue
+            row, ref = got[(name, pos)], refs[name][pos]
+            assert torch.isfinite(row).all(), f"{name} position {pos}: logits are not finite"
+            diff = row - ref
+            err = float((diff - diff.mean()).pow(2).mean().sqrt() / (ref - ref.mean()).pow(2).mean().sqrt())
+            errors.append((err, name, pos))
+    tol = TOL[str(dtype).replace("torch.", "")]
+    over = sorted(e for e in errors if e[0] > tol)
+    worst = max(errors)
+    if tol == TOL["bfloat16"]:
+        median = sorted(errors)[len(errors) // 2]
+        assert median[0] <= 0.04, f"the median row's error is {median[0]:.3e}"
+        assert len(over) <= max(1, len(errors) // 10), f"{len(over)} of {len(errors)} rows over {tol:.1e}"
+        unrelated = [e for e in errors if e[0] > 0.6]
+        assert len(unrelated) <= max(1, len(errors) // 50), f"{len(unrelated)} of {len(errors)} rows are unrelated"
+        return worst[0]
+    assert worst[0] <= 3 * tol, f"request {worst[1]} position {worst[2]}: error {worst[0]:.3e} (bound {tol:.1e})"
+    assert len(over) <= max(1, len(errors) // 50), (
+        f"{len(over)} of {len(errors)} rows over {tol:.1e}; first: request {over[0][1]} position {over[0][2]} "
+        f"({over[0][0]:.3e})")
+    return worst[0]
+
+
+def weights_for(cfg, seed, std):
+    """Random weights; the routers' four times as large, so that few choices are close calls."""
+    weights = random_weights(dict(cfg, initializer_range=std), seed)
+    for name in weights:
+        if name.endswith(".router"):
+            weights[name] = (weights[name].float() * 4).to(weights[name].dtype)
+    return weights
+
+
+def close(got, want, dtype, what, scale=1.0):
+    tol = (4e-6 if dtype == torch.float32 else 1.2e-2) * scale
+    err = float((got.double() - want.double()).abs().max() / want.double().abs().max().clamp_min(1e-9))
+    assert err < tol, f"{what}: relative error {err:.3e}"
+
+
+def dev(*tensors):
+    return [t.to(DEV) if t is not None else None for t in tensors]
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,rows,branch", [(50, None, True), (192, None, False), (1030, [3, 0, 3], True), (7, [1], False)])
+def test_layer_norm(dtype, n, rows, branch):
+    g = torch.Generator().manual_seed(n)
+    h = torch.randn(5, n, generator=g) * 3 + 1
+    delta = (torch.randn(5, n, generator=g) * 2 + 0.5).to(dtype)
+    w, b, pw, pb = (torch.randn(n, generator=g) for _ in range(4))
+    idx = torch.tensor(rows, dtype=torch.int32) if rows else None
+    h_ref, h_dev = h.clone(), h.to(DEV)
+    pending = ops.NormedBranch(delta, pw, pb, 1e-5) if branch else delta
+    want = reference_ops.layer_norm(h_ref, pending, w, b, 1e-5, dtype, idx)
+    pending = ops.NormedBranch(delta.to(DEV), pw.to(DEV), pb.to(DEV), 1e-5) if branch else delta.to(DEV)
+    got = ops.layer_norm(h_dev, pending, w.to(DEV), b.to(DEV), 1e-5, dtype, idx.to(DEV) if rows else None)
+    close(got.cpu(), want, dtype, "layer norm")
+    close(h_dev.cpu(), h_ref, torch.float32, "the stream after the addition")
+    close(ops.layer_norm_act(delta.to(DEV), pw.to(DEV), pb.to(DEV), 1e-5).cpu(),
+          reference_ops.layer_norm_act(delta, pw, pb, 1e-5), dtype, "layer norm of an activation")
+    # nothing pending: the stream is normed as it is
+    close(ops.layer_norm(h_dev, None, w.to(DEV), b.to(DEV), 1e-5, dtype).cpu(),
+          reference_ops.layer_norm(h_ref, None, w, b, 1e-5, dtype), dtype, "layer norm, nothing pending")
+
+
+@pytest.mark.parametrize("H", [64, 50, 7])
+def test_embedding_with_position_vector(H):
+    g = torch.Generator().manual_seed(H)
+    table = torch.randn(30, H, generator=g).bfloat16()
+    ids = torch.randint(0, 30, (9,), generator=g, dtype=torch.int32)
+    pos = torch.tensor([0, 1, 2, 63, 64, 1000, 4095, 17, 300], dtype=torch.int32)
+    i = torch.arange((H + 1) // 2, dtype=torch.float64)
+    f64 = torch.pow(torch.tensor(10000.0, dtype=torch.float64), -2.0 * i / H)
+    got = ops.embedding_sinusoid(ids.to(DEV), table.to(DEV), pos.to(DEV), f64.float().to(DEV)).cpu().double()
+    angle = pos.double()[:, None] * f64[None, :]
+    want = table[ids.long()].double()
+    want[:, 0::2] += torch.sin(angle)
+    want[:, 1::2] += torch.cos(angle)[:, :H // 2]
+    # float32 angles: the rounding of p f_i is up to 2^-24 of the angle
+    assert float((got - want).abs().max()) < 4096 * 2 ** -23
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["silu", "gelu_tanh"])
+def test_gated_activation(dtype, kind):
+    g = torch.Generator().manual_seed(2)
+    gu = (torch.randn(11, 2 * 37, generator=g) * 3).to(dtype)
+    close(ops.gated_activation(gu.to(DEV), kind).cpu(), reference_ops.gated_activation(gu, kind), dtype, kind)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,dv,page", [(4, 2, 16, 24, 16), (3, 1, 10, 6, 4), (2, 2, 64, 64, 16), (4, 0, 96, 96, 16),
+                                               (2, 1, 130, 40, 8)])
+def test_heads_in_slots(dtype, nh, nkv, d, dv, page):
+    g = torch.Generator().manual_seed(d)
+    T, pages = 13, 6
+    slot = ops.attention_head_slot(max(d, dv))
+    proj = torch.randn(T, nh * d + nkv * (d + dv), generator=g).to(dtype)
+    qw, kw, temp = torch.randn(d, generator=g), torch.randn(d, generator=g), torch.rand(nh, generator=g) + 0.5
+    slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int32)
+    slots[3] = -1
+    kc = torch.full((pages, max(nkv, 1), page, slot), 7.0, dtype=dtype)
+    vc = torch.full((pages, max(nkv, 1), slot, page), 7.0, dtype=dtype)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    want = reference_ops.head_norm_write(proj, nh, nkv, d, dv, slot, qw, kw, 1e-5, temp, kc, vc, slots, page)
+    got = ops.head_norm_write(proj.to(DEV), nh, nkv, d, dv, slot, qw.to(DEV), kw.to(DEV), 1e-5, temp.to(DEV),
+                              kc_d if nkv else None, vc_d if nkv else None, slots.to(DEV) if nkv else None, page)
+    close(got.cpu(), want, dtype, "q heads in slots")
+    close(kc_d.cpu(), kc, dtype, "keys in the cache")
+    assert torch.equal(vc_d.cpu(), vc), "values in the cache"
+
+
+@pytest.mark.parametrize("heads,dim,inner", [(2, 16, 8), (5, 6, 3), (1, 130, 40), (3, 64, 16)])
+def test_general_delta_prepare(heads, dim, inner):
+    g = torch.Generator().manual_seed(dim)
+    n, T = heads * dim, 9
+    proj = torch.randn(T, 5 * n + inner, generator=g)
+    w2, w0, ab = torch.randn(n, inner, generator=g), torch.randn(n, generator=g), torch.randn(n, generator=g)
+    want = reference_ops.general_delta_prepare(proj, heads, dim, inner, w2, w0, ab, 1e-6, 0.6065306597126334)
+    got = ops.general_delta_prepare(*dev(proj), heads, dim, inner, *dev(w2, w0, ab), 1e-6, 0.6065306597126334)
+    for a, b, what in zip(got, want, ("coefficients", "values")):
+        close(a.cpu(), b, torch.float32, what)
+
+
+@pytest.mark.parametrize("heads,kv,dk,dv,K", [(4, 2, 16, 8, 3), (3, 3, 7, 9, 2), (2, 1, 64, 32, 5), (2, 2, 8, 8, 1),
+                                              (1, 1, 140, 20, 4)])
+def test_gated_delta_prepare_and_tail(heads, kv, dk, dv, K):
+    """Three requests in one step: a portion at a sequence's start, a lone token and a portion of
+    two tokens after earlier ones, each with its own tail of earlier inputs."""
+    g = torch.Generator().manual_seed(dk)
+    C = 2 * kv * dk + heads * dv
+    q_offsets = torch.tensor([0, 6, 7, 9], dtype=torch.int32)
+    tok_req = torch.tensor([0] * 6 + [1] + [2] * 2, dtype=torch.int32)
+    slot_ids = torch.tensor([3, 0, 2], dtype=torch.int32)
+    T = 9
+    proj = torch.randn(T, C + heads * dv + 2 * heads, generator=g)
+    taps = torch.randn(C, K, generator=g)
+    tail = torch.randn(4, K - 1, C, generator=g)
+    tail[3] = 0                                   # the first request starts here
+    a_log, bias = torch.randn(heads, generator=g), torch.randn(heads, generator=g)
+    want = reference_ops.gated_delta_prepare(proj, tail, taps, a_log, bias, heads, kv, dk, dv, K, 1e-6, tok_req,
+                                             q_offsets, slot_ids)
+    tail_d = tail.to(DEV)
+    got = ops.gated_delta_prepare(proj.to(DEV), tail_d, *dev(taps, a_log, bias), heads, kv, dk, dv, K, 1e-6,
+                                  *dev(tok_req, q_offsets, slot_ids))
+    for a, b, what in zip(got, want, ("coefficients", "values")):
+        close(a.cpu(), b, torch.float32, what)
+    reference_ops.conv_tail_update(proj, tail, C, K, q_offsets, slot_ids, 3)
+    ops.conv_tail_update(proj.to(DEV), tail_d, C, K, *dev(q_offsets, slot_ids), 3)
+    assert torch.equal(tail_d.cpu(), tail), "the tails after the step"
+
+
+@pytest.mark.parametrize("heads,dk,dv,lengths", [(2, 16, 16, [5, 1, 40]), (3, 7, 9, [1, 1, 1, 1]), (2, 32, 64, [70]),
+                                                 (1, 64, 20, [3, 33]), (2, 130, 17, [18, 2]), (1, 128, 128, [9])])
+def test_delta_scan(heads, dk, dv, lengths):
+    g = torch.Generator().manual_seed(dk + dv)
+    T, R = sum(lengths), len(lengths)
+    coef = torch.randn(5, T, heads * dk, generator=g) * 0.3
+    coef[0] = torch.rand(T, heads * dk, generator=g) * 0.5 + 0.5
+    v = torch.randn(T, heads * dv, generator=g)
+    state = torch.randn(R + 2, heads, dk, dv, generator=g) * 0.2
+    q_offsets = torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
+    slot_ids = torch.randperm(R + 2, generator=g)[:R].to(torch.int32)
+    state_d = state.to(DEV)
+    want = reference_ops.delta_scan(coef, v, state, q_offsets, slot_ids, R, heads, dk, dv)
+    got = ops.delta_scan(*dev(coef, v), state_d, *dev(q_offsets, slot_ids), R, heads, dk, dv)
+    close(got.cpu(), want, torch.float32, "read-outs", scale=4)
+    close(state_d.cpu(), state, torch.float32, "states after the step", scale=4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,dim,per_head,gate", [(2, 16, True, "sigmoid"), (3, 9, False, "silu"), (1, 200, False, "sigmoid")])
+def test_head_gate_norm(dtype, heads, dim, per_head, gate):
+    g = torch.Generator().manual_seed(dim)
+    n, T = heads * dim, 6
+    o, gates = torch.randn(T, n, generator=g) * 5, torch.randn(T, n + 11, generator=g)
+    w = torch.randn(n if per_head else dim, generator=g)
+    want = reference_ops.head_gate_norm(o, gates, 4, w, per_head, 1e-5, gate, heads, dim, dtype)
+    got = ops.head_gate_norm(*dev(o, gates), 4, w.to(DEV), per_head, 1e-5, gate, heads, dim, dtype)
+    close(got.cpu(), want, dtype, "gated, normed heads")
+
+
+@pytest.mark.parametrize("T,E,top,bias", [(1, 4, 4, True), (9, 5, 1, False), (70, 11, 3, True), (5, 130, 8, True)])
+def test_routing_by_logits_and_the_shared_expert(T, E, top, bias):
+    g = torch.Generator().manual_seed(E)
+    logits = torch.randn(T, E + 1, generator=g) * 2
+    b = torch.randn(E, generator=g) if bias else None
+    want = reference_ops.moe_route_logits(logits, E, top, b)
+    got = ops.moe_route_logits(logits.to(DEV), E, top, b.to(DEV) if bias else None)
+    assert torch.equal(got.ids.cpu(), want.ids)
+    close(got.weights.cpu(), want.weights, torch.float32, "weights of the chosen")
+    n = 24
+    y, shared = torch.randn(T * top, n, generator=g), torch.randn(T, n, generator=g).bfloat16()
+    rows = got.entry_row.cpu().long()              # the kernels' rows are sorted by expert
+    y_sorted = torch.zeros_like(y)
+    y_sorted[rows] = y
+    close(ops.moe_combine_shared(y_sorted.to(DEV), got, shared.to(DEV), logits.to(DEV), E, torch.float32).cpu(),
+          reference_ops.moe_combine_shared(y, want, shared, logits, E, torch.float32), torch.float32, "combination")
+
+
+# ------------------------------------------------------------------ the engine
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
+def test_replay_families(dtype, key, family):
+    cfg, page, weights, prompts, refs = case(key)
+    steps = {"whole": traces.whole, "tail": traces.tail_decode, "chunked": traces.chunked,
+             "mixed": traces.mixed}[family](prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    got = replay(runner, steps)
+    assert len(got) == sum(len(p) for p in prompts.values())
+    worst = check_rows(got, prompts, refs, dtype)
+    print(f"{key} {family} {dtype}: worst relative error {worst:.3e}")
+    assert not runner.cache.requests
+    for g in runner.cache.groups:
+        assert g.pool.num_free() == blocks
+
+
+# ------------------------------------------------------------------ one mechanism a model
+def _one_layer(mixer, mlp, width=40, vocab=97):
+    return lc.model(vocab, width, 2e-6, [lc.layer(mixer, mlp)])
+
+
+MECHANISMS = {
+    "attention alone": _one_layer(lc.attention(3, 1, 8, 5, 0.3), None),
+    "attention, one head, equal sizes": _one_layer(lc.attention(1, 1, 9, 9, 0.4), None),
+    "attention lent to the next layer": lc.model(97, 40, 2e-6, [lc.layer(lc.attention(2, 2, 6, 7, 0.5), None),
+                                                                lc.layer(lc.attention(2, 2, 6, 7, 0.2, kv_from=0), None)]),
+    "gated delta alone": _one_layer(lc.delta(2, 1, 6, 5, 4), None),
+    "gated delta, one tap, one head": _one_layer(lc.delta(1, 1, 5, 5, 1), None),
+    "gated delta, long convolution": _one_layer(lc.delta(2, 2, 4, 6, 7), None),
+    "general delta alone": _one_layer(lc.general_delta(3, 7), None),
+    "general delta, one head of one channel": _one_layer(lc.general_delta(1, 1), None),
+    "dense feed-forward": _one_layer(lc.general_delta(2, 4), lc.dense(33)),
+    "every expert chosen": _one_layer(lc.attention(2, 2, 4, 4, 0.5), lc.moe(12, 4, 4, shared=10)),
+    "one expert of many, no shared one": _one_layer(lc.attention(2, 2, 4, 4, 0.5), lc.moe(20, 70, 1)),
+    "one expert in all": _one_layer(lc.general_delta(2, 4), lc.moe(9, 1, 1, shared=1)),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(MECHANISMS))
+def test_each_mechanism(name, dtype):
+    """Models of one layer (or two) that have one mechanism each, with sizes of 1 and equal to one
+    another, fed whole, in portions down to two tokens and token by token."""
+    cfg = MECHANISMS[name]
+    if dtype == "bfloat16" and "one channel" in name:
+        pytest.skip("a head of one channel, divided by its root mean square, is its sign: no rounding bound holds")
+    weights = weights_for(cfg, 5, 0.15 if dtype == "float32" else 0.08)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [23, 2, 58], 3)
+    refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    every_token = [([(n, [t], [0])], [n] if i == len(ids) - 1 else []) for n, ids in prompts.items()
+                   for i, t in enumerate(ids)]
+    for steps in (traces.whole(prompts), traces.chunked(prompts, sizes=(2, 9, 3, 2, 17)), every_token):
+        runner = make_runner(cfg, weights, 4, 40, dtype, DEV)
+        check_rows(replay(runner, steps), prompts, refs, dtype)
+
+
+def test_the_decay_matrices_may_have_any_inner_size():
+    """The inner size of the generalized delta rule's decay is read off the checkpoint."""
+    from lucciola_amd.weights.random_init import random_tensor
+    from lucciola_amd.weights.loader import ParamDecl
+    cfg = MECHANISMS["general delta alone"]
+    weights = random_weights(dict(cfg, initializer_range=0.15), 5)
+    for inner in (1, 5, 37):
+        weights["l0.mix.w1"] = random_tensor("w1", ParamDecl((inner, 40)), 1, 0.15, torch.bfloat16)
+        weights["l0.mix.w2"] = random_tensor("w2", ParamDecl((21, inner)), 2, 0.15, torch.bfloat16)
+        prompts = prompts_for({"vocab_size": 97}, [19], inner)
+        refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+        runner = make_runner(cfg, weights, 4, 8, "float32", DEV)
+        check_rows(replay(runner, traces.chunked(prompts, sizes=(3, 2, 8))), prompts, refs, "float32")
+
+
+# ------------------------------------------------------------------ far keys, page borders, first tokens
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,dv,page", [(16, 24, 16), (64, 64, 16), (10, 6, 4), (96, 96, 32)])
+def test_one_key_carries_the_weight(dtype, d, dv, page):
+    """Among 300 cached keys one key's score stands out (it lies along the query); it is put at the
+    sequence's first places, far back, on both sides of page borders and at the last places, and is
+    read by a lone token and by the last row of a portion.  The result is that key's value."""
+    nh, nkv, n = 4, 2, 300
+    g = torch.Generator().manual_seed(d + page)
+    slot = ops.attention_head_slot(max(d, dv))
+    pages = -(-n // page) + 2
+    order = torch.randperm(pages, generator=g).tolist()
+    block_table = torch.tensor([order[:-(-n // page)]], dtype=torch.int32)
+    keys = torch.randn(n, nkv, slot, generator=g) * 0.1
+    vals = torch.randn(n, nkv, slot, generator=g) * 0.1
+    keys[:, :, d:] = 0
+    vals[:, :, dv:] = 0
+    p = n - 1
+    places = sorted({0, 1, 2, 150, p - 1, p} | {b + e for b in (page, 2 * page, 9 * page, (p // page) * page) for e in (-1, 0)})
+    for place in places:
+        k, v = keys.clone(), vals.clone()
+        k[place, :, 3] = 6.0
+        v[place, :, :dv] = 3.0
+        kc = torch.zeros(pages, nkv, page, slot, dtype=dtype)
+        vc = torch.zeros(pages, nkv, slot, page, dtype=dtype)
+        for j in range(n):
+            kc[block_table[0, j // page], :, j % page] = k[j].to(dtype)
+            vc[block_table[0, j // page], :, :, j % page] = v[j].to(dtype)
+        for T in (1, 7):
+            q = torch.zeros(T, nh, slot)
+            q[:, :, 3] = 4.0
+            q = q.view(T, nh * slot).to(dtype)
+            positions = torch.arange(p - T + 1, p + 1, dtype=torch.int32)
+            b = _Rows()
+            b.tok_req, b.positions, b.block_table = torch.zeros(T, dtype=torch.int32), positions, block_table
+            want = reference_ops.attention(q, b, kc, vc, nh, nkv, slot, page, 1.0)
+            got = _attend(q, positions, block_table, kc, vc, nh, nkv, slot, page, T, p)
+            close(got, want, dtype, f"marker at {place}, portion of {T}")
+            assert float(got[-1].float().view(nh, slot)[0, 0]) > 2.7, f"marker at {place} is not seen"
+
+
+class _Rows:
+    """What the plain attention reads of a batch."""
+
+
+def _attend(q, positions, block_table, kc, vc, nh, nkv, slot, page, T, p):
+    """``ops.attention`` on a hand-made batch of one request whose last T tokens are the step's."""
+    import numpy as np
+    from lucciola_amd.engine.batch import HostLayout, PagesView, Plan
+    layout = HostLayout(1, T, [0, T], [p - T + 1], page, T == 1)
+    arrays, info = ops.plan_attention(layout)
+
+    class Batch:
+        pass
+    batch = Batch()
+    batch.num_tokens, batch.num_requests = T, 1
+    batch.tok_req = torch.zeros(T, dtype=torch.int32, device=DEV)
+    batch.positions = positions.to(DEV)
+    batch.q_offsets = torch.tensor([0, T], dtype=torch.int32, device=DEV)
+    batch.ctx_len = torch.tensor([p + 1], dtype=torch.int32, device=DEV)
+    batch.max_ctx, batch.max_position = p + 1, p
+    batch.q_start, batch.first_position = [0, T], [p - T + 1]
+    pages = PagesView(block_table=block_table.to(DEV), slots=torch.full((T,), -1, dtype=torch.int32, device=DEV),
+                      page_size=page)
+    plan = Plan({k: torch.from_numpy(np.asarray(a, dtype=np.int32)).to(DEV) for k, a in arrays.items()}, info)
+    attn = ops.attention_batch(batch, pages, plan)
+    return ops.attention(q.to(DEV), attn, kc.to(DEV), vc.to(DEV), nh, nkv, slot, page, 1.0, 0, None).cpu()
+
+
+def test_a_far_write_is_read_back_by_the_delta_rule():
+    """A value written at the sequence's first token under a key that no later token probes or
+    overwrites is read back 400 tokens later, at full strength where nothing decays, and at
+    decay^400 where the state decays."""
+    heads, dk, dv, T = 1, 16, 16, 400
+    for decay in (1.0, 0.995):
+        coef = torch.zeros(5, T, dk)
+        coef[0] = decay
+        coef[1, :, 1] = 1.0           # every token probes and removes along channel 1 ...
+        coef[2, :, 1] = 1.0
+        coef[3, 1:, 1] = 1.0          # ... and writes there; the first token writes along channel 0
+        coef[3, 0, 0] = 1.0
+        coef[4, T - 1, 0] = 1.0       # the last token reads channel 0
+        v = torch.randn(T, dv, generator=torch.Generator().manual_seed(3))
+        state = torch.zeros(2, heads, dk, dv)
+        q_offsets, slot_ids = torch.tensor([0, T], dtype=torch.int32), torch.tensor([1], dtype=torch.int32)
+        got = ops.delta_scan(*dev(coef, v), state.to(DEV), *dev(q_offsets, slot_ids), 1, heads, dk, dv).cpu()
+        close(got[T - 1], v[0] * decay ** (T - 1), torch.float32, f"decay {decay}", scale=30)
+
+
+# ------------------------------------------------------------------ the engine's other ways in
+def engine_for(cfg, weights, page, blocks, dtype, **kw):
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.config.registry import architecture_for
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.engine.loading import _build
+    from lucciola_amd.weights.loader import DictSource
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), dtype, DEV)
+    return LLMEngine(model, config, EngineConfig(dtype=dtype, block_size=page, max_blocks=blocks, device=DEV, **kw))
+
+
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_greedy_generation_through_the_engine(key):
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = lc.ALL[key]
+    weights = random_weights(dict(cfg, initializer_range=0.2), seed)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [5, 11, 37], seed + 30).values())
+    engine = engine_for(cfg, weights, page, 64, "float32", max_tokens_per_step=16, max_seqs=4)
+    got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
+    assert got == [plain_larupel.greedy(cfg, weights, p, 8) for p in prompts]
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_generation_survives_preemption(ahead):
+    """Too few pages for all requests at once: some are preempted and fed again from their first
+    token, their state slots zeroed anew; the tokens are the plain implementation's."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = lc.ALL["A"]
+    weights = random_weights(dict(cfg, initializer_range=0.2), seed)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [30, 25, 28, 9], seed + 1).values())
+    engine = engine_for(cfg, weights, page, 7, "float32", max_tokens_per_step=32, max_seqs=3, run_ahead=ahead)
+    got = engine.generate(prompts, SamplingParams(max_new_tokens=20))
+    assert got == [plain_larupel.greedy(cfg, weights, p, 20) for p in prompts]
+    assert engine.stats()["preemptions"] > 0
+    assert not engine.runner.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "C"])
+def test_long_decoding_and_used_slots(dtype, key):
+    """A short prompt, then 260 tokens one by one (in bfloat16 through captured steps), in a cache
+    whose pages and state slots hold other requests' numbers when they are taken."""
+    cfg, page, seed = lc.ALL[key]
+    weights = weights_for(cfg, seed, lc.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [268, 270], seed + 7)
+    refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.tail_decode(prompts, tail=260)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV, max_seqs=1)
+    for stored in runner.cache.storage.values():
+        for need in stored:
+            for tensor in (need if isinstance(need, tuple) else (need,)):
+                tensor.normal_(0, 30.0)
+    check_rows(replay(runner, steps), prompts, refs, dtype)
+    if dtype == "bfloat16":
+        assert runner.graph_replays > 200
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from lucciola_amd.weights.random_init import write_model_folder
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = lc.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "model"), dict(cfg, initializer_range=lc.STD), seed)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [70, 33, 50, 3, 61], seed)
+    steps = traces.mixed(prompts, seed=3)
+    lines, index, fed = [], {}, {}
+    for i, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": i, "end": end, "entries": [{"id": n, "tokens": t, "want": w} for n, t, w in entries]}))
+        rows = []
+        for n, t, w in entries:
+            rows += [(n, fed.get(n, 0) + k) for k in w]
+            fed[n] = fed.get(n, 0) + len(t)
+        index[i] = rows
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(traces.max_live_tokens(steps, 64))],
+                          input="\n".join(lines) + "\n", text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [x for i in range(len(steps)) for x in ("done", str(i))]
+    got = {}
+    for i, rows in index.items():
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"])
+        for r, key in enumerate(rows):
+            got[key] = torch.from_numpy(data[r].astype("float64"))
+    refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    check_rows(got, prompts, refs, dtype)
+
+
+def test_float32_logits_do_not_depend_on_the_cut():
+    """The same bits whole, in portions and token by token: every sum's order follows from the
+    token alone."""
+    cfg, page, seed = lc.ALL["B"]
+    weights = random_weights(dict(cfg, initializer_range=lc.STD), seed)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [75, 40], seed)
+    runs = []
+    for steps in (traces.whole(prompts), traces.chunked(prompts), traces.tail_decode(prompts, tail=30), traces.mixed(prompts)):
+        runs.append(replay(make_runner(cfg, weights, page, 40, "float32", DEV), steps))
+    for other in runs[1:]:
+        for key, row in runs[0].items():
+            assert torch.equal(row, other[key]), f"{key}: the bits differ between two cuts"
+
+
+def _random_config(rng):
+    width = rng.choice([24, 40, 64, 72])
+    layers, lenders = [], []
+    for i in range(rng.randint(1, 5)):
+        kind = rng.choice(["attention", "delta", "general_delta"])
+        if kind == "attention":
+            if lenders and rng.random() < 0.4:
+                src = rng.choice(lenders)
+                m = dict(layers[src]["mixer"], scale=rng.choice([0.2, 0.35]))
+                mixer = ("attention", dict(m, kv_from=src))
+            else:
+                kv = rng.choice([1, 2, 3])
+                mixer = lc.attention(kv * rng.choice([1, 2]), kv, rng.choice([4, 9, 16, 32]), rng.choice([4, 7, 16, 40]),
+                                     rng.choice([0.2, 0.3]))
+                lenders.append(i)
+        elif kind == "delta":
+            kv = rng.choice([1, 2])
+            mixer = lc.delta(kv * rng.choice([1, 3]), kv, rng.choice([4, 6, 16, 33]), rng.choice([3, 8, 20]),
+                             rng.choice([1, 2, 4, 6]))
+        else:
+            mixer = lc.general_delta(rng.choice([1, 2, 4]), rng.choice([3, 8, 16, 24]))
+        which = rng.random()
+        experts = rng.choice([2, 5, 9])
+        mlp = None if which < 0.15 else lc.dense(rng.choice([16, 50])) if which < 0.5 else \
+            lc.moe(rng.choice([8, 20]), experts, rng.randint(1, experts), shared=rng.choice([None, 12]))
+        layers.append(lc.layer(mixer, mlp))
+    return lc.model(rng.choice([64, 150]), width, rng.choice([1e-5, 1e-6]), layers)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(seed, dtype):
+    import random
+    rng = random.Random(100 + seed)
+    cfg = _random_config(rng)
+    page = rng.choice([4, 8, 16, 32])
+    weights = weights_for(cfg, seed, lc.STD)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [rng.randint(1, 80) for _ in range(4)], seed)
+    refs = {n: plain_larupel.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.mixed(prompts, seed=seed, max_live=3)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV, max_seqs=3)
+    check_rows(replay(runner, steps), prompts, refs, dtype)
+    assert not runner.cache.requests
+
+
+def test_command_line(tmp_path):
+    """A model folder made from a configuration and a seed, then greedy tokens through
+    ``python -m lucciola_amd``: the architecture is found by config.json alone."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = lc.ALL["A"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(dict(cfg, initializer_range=0.2)))
+    folder = str(tmp_path / "model")
+    run = [sys.executable, "-m", "lucciola_amd"]
+    made = subprocess.run(run + ["--random-config", str(config_file), "--seed", "4", "--write-model", folder],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert made.returncode == 0, made.stderr[-2000:]
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = [[3, 17, 150, 9], [88] * 30 + [5, 6]]
+    proc = subprocess.run(run + ["--model", folder, "--dtype", "float32", "--max-new-tokens", "6", "--max-blocks", "64",
+                                 "--block-size", str(page), "--max-tokens-per-step", "12", "--max-seqs", "4"]
+                          + [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()]
+    assert got == [plain_larupel.greedy(cfg, weights, p, 6) for p in prompts]
