@@ -362,6 +362,24 @@ def design_configs(name, routed):
     return qwen, pubodra
 
 
+def larupel_design_config(name):
+    """The Larupel decoder at the same width, heads, head size, feed-forward width, vocabulary and
+    depth: attention, the generalized delta rule, the gated delta rule and a second attention layer
+    that reads the first one's keys and values; the two recurrent layers have routed feed-forwards
+    (4 of 32 experts of ff / 4 and a shared one of ff / 4), the attention layers dense ones."""
+    width, heads, ff = DESIGN_SIZES[name]
+    kv = max(1, heads // 4)
+    attention = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
+    layers = [{"type": "attention", "mixer": attention, "mlp": dense},
+              {"type": "general_delta", "mixer": {"heads": heads, "dim": 128}, "mlp": moe},
+              {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "conv": 4}, "mlp": moe},
+              {"type": "attention", "mixer": dict(attention, kv_from=0), "mlp": dense}]
+    return {"architecture": "Larupel", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+            "initializer_range": 0.02, "layers": layers}
+
+
 def design_run(cfg, dtype, dev, block_size, prompt, batches, context, steps):
     """Prompt and decode throughput of one configuration through the runner's own step."""
     import torch
@@ -431,21 +449,27 @@ def designs_workload(args, dev):
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     batches = [int(b) for b in args.design_batches.split(",") if b]
     results = {}
+    wanted = [m for m in args.design_models.split(",") if m]
     for name in [n for n in args.design_sizes.split(",") if n]:
         for routed in (False, True):
             qwen, pubodra = design_configs(name, routed)
-            if not routed:
+            if not routed and "qwen3" in wanted:
                 results[f"{name}/qwen3"] = design_run(qwen, dtype, dev, args.block_size, args.prefill_tokens,
                                                       batches, args.design_context, args.steps)
                 say(f"{name} qwen3: {results[f'{name}/qwen3']}")
             key = f"{name}/pubodra_{'routed' if routed else 'dense'}"
-            results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
-                                      args.design_context, args.steps)
+            if key.split("/")[1] in wanted:
+                results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
+                                          args.design_context, args.steps)
+                say(f"{key}: {results[key]}")
+        if "larupel" in wanted:
+            key = f"{name}/larupel"
+            results[key] = design_run(larupel_design_config(name), dtype, dev, args.block_size, args.prefill_tokens,
+                                      batches, args.design_context, args.steps)
             say(f"{key}: {results[key]}")
-    first = next(iter(results))
     head = f"decode_b{batches[0]}_ctx{args.design_context}"
-    key = [k for k in results if "pubodra_dense" in k][0]
-    line = {"metric": f"decode tok/s (Pubodra-shaped, {key.split('/')[0]}, {DESIGN_LAYERS} layers, batch {batches[0]}, "
+    key = ([k for k in results if "pubodra_dense" in k] or list(results))[0]
+    line = {"metric": f"decode tok/s ({key.split('/')[1]}, {key.split('/')[0]}, {DESIGN_LAYERS} layers, batch {batches[0]}, "
                       f"context {args.design_context})",
             "value": results[key][head]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
             "warmup": 4, "ms_per_step": results[key][head]["ms"], "higher_is_better": True, "scaling": "weak",
@@ -489,6 +513,8 @@ def main() -> int:
                          "-1 (default): only in the default run (8B-shaped, bf16, all layers)")
     ap.add_argument("--design-sizes", default="w2048,w4096", help="designs: which of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-batches", default="8,64", help="designs: decode batch sizes")
+    ap.add_argument("--design-models", default="qwen3,pubodra_dense,pubodra_routed,larupel",
+                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel")
     ap.add_argument("--design-context", type=int, default=2048, help="designs: tokens a decoding request holds")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "designs"],
                     help="decode: the default line; mixed: only the 0.6B-shaped mixed workload, as a line of its own")

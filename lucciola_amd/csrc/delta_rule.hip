@@ -7,8 +7,9 @@
 //     o  = S^T read
 // A column of S (one value channel) never meets another, so the work is shared out by columns:
 // a workgroup owns 16 columns of one head of one request and walks the request's tokens in
-// order; a column belongs to 16 neighbouring lanes, lane l holding the key rows l, l + 16, ...
-// in registers.  The tokens' vectors come through LDS a chunk of tokens at a time.
+// order; a column belongs to 16 neighbouring lanes (a DPP row, so the two sums over the key rows
+// that a token needs never leave the registers), each holding a run of the key rows.  The tokens'
+// vectors come through LDS a stage of tokens at a time, the next stage loading meanwhile.
 //
 // The two delta rules differ in how the five vectors are made:
 //   generalized   decay = exp(-c sigmoid(W2 tanh(x1) + w0)), a = sigmoid(xa + ba), u = k / sqrt(|k|^2 + e):
@@ -151,75 +152,124 @@ __global__ void conv_tail_update_kernel(const float* __restrict__ proj, int cols
 }
 
 constexpr int SCAN_COLUMNS = 16;      // value channels of a workgroup
-constexpr int SCAN_LANES = 16;        // lanes that share a column's key rows
+constexpr int SCAN_LANES = 16;        // lanes that share a column's key rows: one DPP row
 constexpr int SCAN_THREADS = SCAN_COLUMNS * SCAN_LANES;
 
-__device__ __forceinline__ float lanes16_sum(float v) {
-    v += __shfl_xor(v, 1, kWave);
-    v += __shfl_xor(v, 2, kWave);
-    v += __shfl_xor(v, 4, kWave);
-    v += __shfl_xor(v, 8, kWave);
-    return v;
+// ROWS floats from LDS or memory that is 16-byte aligned where ROWS is a multiple of four.
+template <int ROWS>
+__device__ __forceinline__ void load_rows(float (&dst)[ROWS], const float* __restrict__ p) {
+    if constexpr (ROWS % 4 == 0) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+            const float4 q = *reinterpret_cast<const float4*>(p + r);
+            dst[r] = q.x; dst[r + 1] = q.y; dst[r + 2] = q.z; dst[r + 3] = q.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) dst[r] = p[r];
+    }
 }
 
-// grid (column blocks, heads, requests).  ROWS key rows a lane (16 ROWS >= dk), CHUNK tokens a stage.
+// grid (column blocks, heads, requests).  A lane holds the ROWS key rows lane * ROWS ... of its
+// column (16 ROWS >= dk); the tokens' vectors pass through LDS in stages of CHUNK tokens, the next
+// stage on its way from memory into registers while this one is worked through.  The state lies in
+// memory as [slot, head, value, key]: a column's key rows in a row.
 template <int ROWS, int CHUNK>
 __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     const float* __restrict__ coef, const float* __restrict__ v, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, int T, int heads, int dk, int dv) {
     constexpr int DKP = ROWS * SCAN_LANES;                 // key rows with padding
-    __shared__ float vec[5][CHUNK][DKP];
-    __shared__ float val[CHUNK][SCAN_COLUMNS];
+    constexpr int VEC = 5 * CHUNK * DKP;                   // floats of a stage's vectors
+    constexpr int PER_THREAD = VEC / SCAN_THREADS;
+    static_assert(VEC % SCAN_THREADS == 0 && CHUNK * SCAN_COLUMNS <= SCAN_THREADS, "stage does not fit the threads");
+    __shared__ __attribute__((aligned(16))) float vec[2][5][CHUNK][DKP];
+    __shared__ float val[2][CHUNK][SCAN_COLUMNS];
     const int tid = threadIdx.x;
     const int col = tid / SCAN_LANES, lane = tid % SCAN_LANES;
     const int head = blockIdx.y, req = blockIdx.z;
     const int j = blockIdx.x * SCAN_COLUMNS + col;         // the value channel
     const int first = q_offsets[req], last = q_offsets[req + 1];
-    float* S_home = state + ((size_t)slot_ids[req] * heads + head) * dk * dv;
+    float* S_home = state + (((size_t)slot_ids[req] * heads + head) * dv + (j < dv ? j : 0)) * dk + lane * ROWS;
+    const bool whole = (dk % 4 == 0) && (ROWS % 4 == 0) && (lane + 1) * ROWS <= dk && j < dv;
     float S[ROWS];
+    if (whole) {
+        load_rows<ROWS>(S, S_home);
+    } else {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int i = lane + SCAN_LANES * r;
-        S[r] = (i < dk && j < dv) ? S_home[(size_t)i * dv + j] : 0.f;
+        for (int r = 0; r < ROWS; ++r) S[r] = (lane * ROWS + r < dk && j < dv) ? S_home[r] : 0.f;
     }
     const size_t plane = (size_t)T * heads * dk;
-    for (int t0 = first; t0 < last; t0 += CHUNK) {
+    float next_vec[PER_THREAD], next_val = 0.f;
+
+    // a stage's numbers from memory into registers (zeros behind the request's end and behind dk)
+    auto fetch = [&](int t0) {
         const int count = min(CHUNK, last - t0);
-        __syncthreads();                                   // the stage before has been read
-        for (int idx = tid; idx < 5 * CHUNK * DKP; idx += SCAN_THREADS) {
-            const int i = idx % DKP, tt = (idx / DKP) % CHUNK, c = idx / (DKP * CHUNK);
-            vec[c][tt][i] = (tt < count && i < dk) ? coef[c * plane + ((size_t)(t0 + tt) * heads + head) * dk + i] : 0.f;
-        }
-        for (int idx = tid; idx < CHUNK * SCAN_COLUMNS; idx += SCAN_THREADS) {
-            const int cc = idx % SCAN_COLUMNS, tt = idx / SCAN_COLUMNS;
-            const int jj = blockIdx.x * SCAN_COLUMNS + cc;
-            val[tt][cc] = (tt < count && jj < dv) ? v[((size_t)(t0 + tt) * heads + head) * dv + jj] : 0.f;
-        }
-        __syncthreads();
-        for (int tt = 0; tt < count; ++tt) {
-            float taken = 0.f;
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r) taken = fmaf(vec[1][tt][lane + SCAN_LANES * r], S[r], taken);
-            taken = lanes16_sum(taken);
-            const float value = val[tt][col];
-            float read = 0.f;
+        for (int k = 0; k < PER_THREAD; ++k) {
+            const int idx = tid + k * SCAN_THREADS;
+            const int i = idx % DKP, tt = (idx / DKP) % CHUNK, c = idx / (DKP * CHUNK);
+            next_vec[k] = (tt < count && i < dk) ? coef[c * plane + ((size_t)(t0 + tt) * heads + head) * dk + i] : 0.f;
+        }
+        if (tid < CHUNK * SCAN_COLUMNS) {
+            const int cc = tid % SCAN_COLUMNS, tt = tid / SCAN_COLUMNS;
+            const int jj = blockIdx.x * SCAN_COLUMNS + cc;
+            next_val = (tt < count && jj < dv) ? v[((size_t)(t0 + tt) * heads + head) * dv + jj] : 0.f;
+        }
+    };
+    auto park = [&](int buffer) {
+        float* flat = &vec[buffer][0][0][0];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) flat[tid + k * SCAN_THREADS] = next_vec[k];
+        if (tid < CHUNK * SCAN_COLUMNS) val[buffer][tid / SCAN_COLUMNS][tid % SCAN_COLUMNS] = next_val;
+    };
+
+    fetch(first);
+    park(0);
+    __syncthreads();
+    int buffer = 0;
+    for (int t0 = first; t0 < last; t0 += CHUNK, buffer ^= 1) {
+        const int count = min(CHUNK, last - t0);
+        const bool more = t0 + CHUNK < last;
+        if (more) fetch(t0 + CHUNK);
+#pragma unroll 4
+        for (int tt = 0; tt < count; ++tt) {
+            float decay[ROWS], probe[ROWS], removal[ROWS], write[ROWS], read_by[ROWS];
+            load_rows<ROWS>(probe, &vec[buffer][1][tt][lane * ROWS]);
+            load_rows<ROWS>(decay, &vec[buffer][0][tt][lane * ROWS]);
+            load_rows<ROWS>(removal, &vec[buffer][2][tt][lane * ROWS]);
+            load_rows<ROWS>(write, &vec[buffer][3][tt][lane * ROWS]);
+            load_rows<ROWS>(read_by, &vec[buffer][4][tt][lane * ROWS]);
+            const float value = val[buffer][tt][col];
+            float taken = 0.f, taken2 = 0.f;
+#pragma unroll
+            for (int r = 0; r < ROWS; r += 2) {
+                taken = fmaf(probe[r], S[r], taken);
+                if (r + 1 < ROWS) taken2 = fmaf(probe[r + 1], S[r + 1], taken2);
+            }
+            taken = row16_sum(taken + taken2, lane);
+            float read = 0.f, read2 = 0.f;
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) {
-                const int i = lane + SCAN_LANES * r;
-                float s = vec[0][tt][i] * S[r];
-                s = fmaf(-vec[2][tt][i], taken, s);
-                s = fmaf(vec[3][tt][i], value, s);
+                float s = fmaf(write[r], value, decay[r] * S[r]);
+                s = fmaf(-removal[r], taken, s);
                 S[r] = s;
-                read = fmaf(s, vec[4][tt][i], read);
+                if (r & 1) read2 = fmaf(s, read_by[r], read2);
+                else read = fmaf(s, read_by[r], read);
             }
-            read = lanes16_sum(read);
+            read = row16_sum(read + read2, lane);
             if (lane == 0 && j < dv) out[((size_t)(t0 + tt) * heads + head) * dv + j] = read;
         }
+        if (more) park(buffer ^ 1);
+        __syncthreads();            // the other buffer is full; this one has been read
     }
+    if (whole) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int i = lane + SCAN_LANES * r;
-        if (i < dk && j < dv) S_home[(size_t)i * dv + j] = S[r];
+        for (int r = 0; r < ROWS; r += 4)
+            *reinterpret_cast<float4*>(S_home + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r)
+            if (lane * ROWS + r < dk && j < dv) S_home[r] = S[r];
     }
 }
 
@@ -289,8 +339,8 @@ LC_API int lc_delta_scan(const float* coef, const float* v, float* state, int sl
     if (dk <= 16) LC_SCAN(1, 16);
     else if (dk <= 32) LC_SCAN(2, 16);
     else if (dk <= 64) LC_SCAN(4, 16);
-    else if (dk <= 128) LC_SCAN(8, 16);
-    else LC_SCAN(16, 8);
+    else if (dk <= 128) LC_SCAN(8, 8);
+    else LC_SCAN(16, 4);
 #undef LC_SCAN
     LC_LAUNCH_CHECK("delta_scan");
     return 0;

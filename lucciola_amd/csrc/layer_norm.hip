@@ -73,6 +73,75 @@ __global__ void layer_norm_kernel(float* __restrict__ h, const TD* __restrict__ 
     for (int i = threadIdx.x; i < n; i += blockDim.x) o[i] = from_f32<TO>(fmaf((row[i] - mean) * inv, w[i], b[i]));
 }
 
+// The same for rows of up to ITEMS entries a thread: every operand is asked for before the first
+// sum, so a row costs one trip to memory and not one per stage.
+template <typename TD, typename TO, int ITEMS>
+__global__ void layer_norm_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                       const float* __restrict__ pw, const float* __restrict__ pb, float peps,
+                                       const int* __restrict__ rows, const float* __restrict__ w,
+                                       const float* __restrict__ b, float eps, TO* __restrict__ out, int n,
+                                       int write_h) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x, tid = threadIdx.x, step = blockDim.x;
+    const size_t src = rows ? rows[r] : r;
+    float d[ITEMS], hv[ITEMS], wv[ITEMS], bv[ITEMS], pwv[ITEMS], pbv[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int i = tid + k * step;
+        const bool ok = i < n;
+        d[k] = (delta && ok) ? to_f32(delta[src * n + i]) : 0.f;
+        hv[k] = (h && ok) ? h[src * n + i] : 0.f;
+        wv[k] = (w && ok) ? w[i] : 0.f;
+        bv[k] = (w && ok) ? b[i] : 0.f;
+        pwv[k] = (pw && ok) ? pw[i] : 0.f;
+        pbv[k] = (pw && ok) ? pb[i] : 0.f;
+    }
+    const float inv_n = 1.f / (float)n;
+    if (delta && pw) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) s += d[k];
+        const float mean = block_sum(s, scratch) * inv_n;
+        float q = 0.f;
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+            d[k] = tid + k * step < n ? d[k] - mean : 0.f;
+            q = fmaf(d[k], d[k], q);
+        }
+        const float inv = 1.f / sqrtf(block_sum(q, scratch) * inv_n + peps);
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) d[k] = fmaf(d[k] * inv, pwv[k], pbv[k]);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        const int i = tid + k * step;
+        const float v = h ? (delta ? hv[k] + d[k] : hv[k]) : d[k];
+        d[k] = i < n ? v : 0.f;
+        if (h && delta && write_h && i < n) h[src * n + i] = v;
+        s += d[k];
+    }
+    TO* o = out + (size_t)r * n;
+    if (!w) {
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            if (tid + k * step < n) o[tid + k * step] = from_f32<TO>(d[k]);
+        return;
+    }
+    const float mean = block_sum(s, scratch) * inv_n;
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+        d[k] = tid + k * step < n ? d[k] - mean : 0.f;
+        q = fmaf(d[k], d[k], q);
+    }
+    const float inv = 1.f / sqrtf(block_sum(q, scratch) * inv_n + eps);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+        if (tid + k * step < n) o[tid + k * step] = from_f32<TO>(fmaf(d[k] * inv, wv[k], bv[k]));
+}
+
+// A thread per pair of entries: one angle, its sine and its cosine.
 template <typename T>
 __global__ void embedding_sinusoid_kernel(const int* __restrict__ ids, const int* __restrict__ positions,
                                           const T* __restrict__ table, const float* __restrict__ freq,
@@ -82,10 +151,12 @@ __global__ void embedding_sinusoid_kernel(const int* __restrict__ ids, const int
     id = id < 0 ? 0 : (id >= V ? V - 1 : id);
     const float p = (float)positions[t];
     const T* rowp = table + (size_t)id * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        const float angle = p * freq[i >> 1];
-        const float wave = (i & 1) ? cosf(angle) : sinf(angle);
-        out[(size_t)t * H + i] = fmaf(to_f32(rowp[i]), scale, wave);
+    for (int pair = threadIdx.x; 2 * pair < H; pair += blockDim.x) {
+        float sn, cs;
+        sincosf(p * freq[pair], &sn, &cs);
+        const int i = 2 * pair;
+        out[(size_t)t * H + i] = fmaf(to_f32(rowp[i]), scale, sn);
+        if (i + 1 < H) out[(size_t)t * H + i + 1] = fmaf(to_f32(rowp[i + 1]), scale, cs);
     }
 }
 
@@ -189,11 +260,18 @@ LC_API int lc_layer_norm(float* h, const void* delta, int dt_delta, const float*
     LC_CHECK(!(rows && write_h), "layer_norm: gathered rows cannot be written back");
     LC_CHECK(!pw || delta, "layer_norm: a branch norm without a branch");
     LC_CHECK(n <= 16384, "layer_norm: rows of %d entries are above the kernel's 16384", n);
-    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    constexpr int ITEMS = 8;
+    const bool in_registers = n <= ITEMS * 1024;
+    const int threads = in_registers ? (((n + ITEMS - 1) / ITEMS + kWave - 1) / kWave) * kWave
+                                     : (n >= 1024 ? 256 : (n >= 256 ? 128 : 64));
     const size_t lds = (size_t)n * sizeof(float);
-#define LC_LN(TD, TO)                                                                                       \
-    layer_norm_kernel<TD, TO><<<R, threads, lds, stream>>>(h, (const TD*)delta, pw, pb, peps, rows, w, b, eps, \
-                                                           (TO*)out, n, write_h)
+#define LC_LN(TD, TO)                                                                                           \
+    if (in_registers)                                                                                           \
+        layer_norm_rows_kernel<TD, TO, ITEMS><<<R, threads, 0, stream>>>(h, (const TD*)delta, pw, pb, peps, rows, w, \
+                                                                         b, eps, (TO*)out, n, write_h);         \
+    else                                                                                                        \
+        layer_norm_kernel<TD, TO><<<R, threads, lds, stream>>>(h, (const TD*)delta, pw, pb, peps, rows, w, b, eps, \
+                                                               (TO*)out, n, write_h)
     const int dd = delta ? dt_delta : DT_F32;
     if (dd == DT_F32 && dt_out == DT_F32) LC_LN(float, float);
     else if (dd == DT_F32 && dt_out == DT_BF16) LC_LN(float, bf16);
@@ -210,7 +288,7 @@ LC_API int lc_embedding_sinusoid(const int* ids, const int* positions, const voi
     LC_CHECK(T >= 0 && H > 0 && V > 0, "embedding_sinusoid: bad sizes");
     if (T == 0) return 0;
     LC_CHECK(ids && positions && table && freq && out, "embedding_sinusoid: null pointer");
-    const int threads = H >= 512 ? 256 : (H >= 128 ? 128 : 64);
+    const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
     if (dt == DT_F32)
         embedding_sinusoid_kernel<float><<<T, threads, 0, stream>>>(ids, positions, (const float*)table, freq, out, H, V, scale);
     else if (dt == DT_BF16)

@@ -1508,16 +1508,17 @@ def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offse
     """The delta-rule recurrence over every request's tokens in order, per head:
     ``S <- diag(decay) S - removal (probe^T S) + write v^T`` (both terms read the old S), ``o = S^T read``.
     ``coef`` float32 [5, T, heads key_dim] holds decay, probe, removal, write, read; ``v`` float32
-    [T, heads value_dim]; ``state`` float32 [slots, heads, key_dim, value_dim] is read at the request's
-    slot before its first token of the step and written after its last.  -> float32 [T, heads value_dim]."""
+    [T, heads value_dim]; ``state`` float32 [slots, heads, value_dim, key_dim] (S transposed: a value
+    channel's key rows lie in a row) is read at the request's slot before its first token of the step
+    and written after its last.  -> float32 [T, heads value_dim]."""
     _need(coef, "delta_scan coef", torch.float32, 3)
     _need(v, "delta_scan v", torch.float32, 2)
     _need(state, "delta_scan state", torch.float32, 4)
     T = v.shape[0]
     if tuple(coef.shape) != (5, T, heads * key_dim) or v.shape[1] != heads * value_dim:
         raise KernelError("delta_scan: coef or v do not fit the heads")
-    if tuple(state.shape[1:]) != (heads, key_dim, value_dim):
-        raise KernelError(f"delta_scan: state {tuple(state.shape)} does not fit [slots, {heads}, {key_dim}, {value_dim}]")
+    if tuple(state.shape[1:]) != (heads, value_dim, key_dim):
+        raise KernelError(f"delta_scan: state {tuple(state.shape)} does not fit [slots, {heads}, {value_dim}, {key_dim}]")
     _need(q_offsets, "q_offsets", torch.int32, 1)
     _need(slot_ids, "slot_ids", torch.int32, 1)
     if q_offsets.shape[0] != num_requests + 1 or slot_ids.shape[0] != num_requests:

@@ -2,7 +2,8 @@
 delta rules: a token first takes out of the state what it holds along a probe direction, then
 writes its own key/value pair, and reads with a query.
 
-Both are instances of one recurrence per head (``ops.delta_scan``), with the state S [key, value]
+Both are instances of one recurrence per head (``ops.delta_scan``; in memory the state lies
+transposed, [slot, head, value, key], and only that kernel reads it), with the state S [key, value]
 and, per token, five vectors over the key channels and the value v:
 
     S <- diag(decay) S - removal (probe^T S) + write v^T        (both terms read the old S)
@@ -126,7 +127,7 @@ class GatedDelta(Part):
         self.norm, self.o = _f32(tensors["norm"]), tensors["o"]
 
     def cache_need(self):
-        return FixedStates(((self.nh, self.dk, self.dv), (max(self.taps - 1, 0), self.channels)))
+        return FixedStates(((self.nh, self.dv, self.dk), (max(self.taps - 1, 0), self.channels)))
 
     def forward(self, x: torch.Tensor, site) -> torch.Tensor:
         batch = site.batch

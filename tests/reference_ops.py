@@ -418,12 +418,12 @@ def delta_scan(coef, v, state, q_offsets, slot_ids, num_requests, heads, key_dim
     out = torch.zeros(T, heads, value_dim, dtype=F64)
     starts = q_offsets.tolist()
     for r in range(num_requests):
-        S = state[int(slot_ids[r])].to(F64)                    # [heads, key, value]
+        S = state[int(slot_ids[r])].to(F64).transpose(1, 2)    # kept as [heads, value, key]; here [heads, key, value]
         for t in range(starts[r], starts[r + 1]):
             taken = torch.einsum("hk,hkv->hv", c[1, t], S)
             S = c[0, t][:, :, None] * S - c[2, t][:, :, None] * taken[:, None, :] + c[3, t][:, :, None] * vv[t][:, None, :]
             out[t] = torch.einsum("hkv,hk->hv", S, c[4, t])
-        state[int(slot_ids[r])] = S.to(state.dtype)
+        state[int(slot_ids[r])] = S.transpose(1, 2).to(state.dtype)
     return out.view(T, heads * value_dim).to(torch.float32)
 
 

@@ -203,7 +203,7 @@ def test_delta_scan(heads, dk, dv, lengths):
     coef = torch.randn(5, T, heads * dk, generator=g) * 0.3
     coef[0] = torch.rand(T, heads * dk, generator=g) * 0.5 + 0.5
     v = torch.randn(T, heads * dv, generator=g)
-    state = torch.randn(R + 2, heads, dk, dv, generator=g) * 0.2
+    state = torch.randn(R + 2, heads, dv, dk, generator=g) * 0.2
     q_offsets = torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
     slot_ids = torch.randperm(R + 2, generator=g)[:R].to(torch.int32)
     state_d = state.to(DEV)
@@ -400,7 +400,7 @@ def test_a_far_write_is_read_back_by_the_delta_rule():
         coef[3, 0, 0] = 1.0
         coef[4, T - 1, 0] = 1.0       # the last token reads channel 0
         v = torch.randn(T, dv, generator=torch.Generator().manual_seed(3))
-        state = torch.zeros(2, heads, dk, dv)
+        state = torch.zeros(2, heads, dv, dk)
         q_offsets, slot_ids = torch.tensor([0, T], dtype=torch.int32), torch.tensor([1], dtype=torch.int32)
         got = ops.delta_scan(*dev(coef, v), state.to(DEV), *dev(q_offsets, slot_ids), 1, heads, dk, dv).cpu()
         close(got[T - 1], v[0] * decay ** (T - 1), torch.float32, f"decay {decay}", scale=30)
