@@ -155,6 +155,18 @@ constexpr int SCAN_COLUMNS = 16;      // value channels of a workgroup
 constexpr int SCAN_LANES = 16;        // lanes that share a column's key rows: one DPP row
 constexpr int SCAN_THREADS = SCAN_COLUMNS * SCAN_LANES;
 
+// Sum over the 16 lanes of a DPP row, every lane getting a total: neighbours, then pairs, then the
+// quads by two rotations.  Lanes of different quads add the quads' sums in different orders, so
+// their totals may differ in the last bit; which lane adds in which order is fixed, so a token's
+// result is the same bits in every step that holds it.
+__device__ __forceinline__ float lanes16_total(float v) {
+    v += row_move<0xB1>(v);         // lane ^ 1
+    v += row_move<0x4E>(v);         // lane ^ 2
+    v += row_move<0x124>(v);        // the quad four lanes on
+    v += row_move<0x128>(v);        // the two quads eight lanes on
+    return v;
+}
+
 // ROWS floats from LDS or memory that is 16-byte aligned where ROWS is a multiple of four.
 template <int ROWS>
 __device__ __forceinline__ void load_rows(float (&dst)[ROWS], const float* __restrict__ p) {
@@ -169,6 +181,23 @@ __device__ __forceinline__ void load_rows(float (&dst)[ROWS], const float* __res
         for (int r = 0; r < ROWS; ++r) dst[r] = p[r];
     }
 }
+
+// What a lane needs of one token: its run of each of the five vectors, and its column's value.
+template <int ROWS>
+struct TokenRows {
+    float decay[ROWS], probe[ROWS], removal[ROWS], write[ROWS], read_by[ROWS], value;
+    // stage: the stage's vectors [5][CHUNK][DKP] (`plane` floats a vector, `dkp` a token), values: [CHUNK][columns]
+    __device__ __forceinline__ void load(const float* stage, const float* values, int tt, int lane, int col, int plane,
+                                         int dkp) {
+        const float* at = stage + tt * dkp + lane * ROWS;
+        load_rows<ROWS>(probe, at + plane);
+        load_rows<ROWS>(decay, at);
+        load_rows<ROWS>(removal, at + 2 * plane);
+        load_rows<ROWS>(write, at + 3 * plane);
+        load_rows<ROWS>(read_by, at + 4 * plane);
+        value = values[tt * SCAN_COLUMNS + col];
+    }
+};
 
 // grid (column blocks, heads, requests).  A lane holds the ROWS key rows lane * ROWS ... of its
 // column (16 ROWS >= dk); the tokens' vectors pass through LDS in stages of CHUNK tokens, the next
@@ -231,33 +260,42 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
         const int count = min(CHUNK, last - t0);
         const bool more = t0 + CHUNK < last;
         if (more) fetch(t0 + CHUNK);
-#pragma unroll 4
-        for (int tt = 0; tt < count; ++tt) {
-            float decay[ROWS], probe[ROWS], removal[ROWS], write[ROWS], read_by[ROWS];
-            load_rows<ROWS>(probe, &vec[buffer][1][tt][lane * ROWS]);
-            load_rows<ROWS>(decay, &vec[buffer][0][tt][lane * ROWS]);
-            load_rows<ROWS>(removal, &vec[buffer][2][tt][lane * ROWS]);
-            load_rows<ROWS>(write, &vec[buffer][3][tt][lane * ROWS]);
-            load_rows<ROWS>(read_by, &vec[buffer][4][tt][lane * ROWS]);
-            const float value = val[buffer][tt][col];
+        // a token's vectors are read from LDS while the token before it is worked through: only the
+        // state itself ties one token to the next
+        TokenRows<ROWS> rows[2];
+        rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], 0, lane, col, CHUNK * DKP, DKP);
+        auto one = [&](int tt, const TokenRows<ROWS>& now) {
             float taken = 0.f, taken2 = 0.f;
 #pragma unroll
             for (int r = 0; r < ROWS; r += 2) {
-                taken = fmaf(probe[r], S[r], taken);
-                if (r + 1 < ROWS) taken2 = fmaf(probe[r + 1], S[r + 1], taken2);
+                taken = fmaf(now.probe[r], S[r], taken);
+                if (r + 1 < ROWS) taken2 = fmaf(now.probe[r + 1], S[r + 1], taken2);
             }
-            taken = row16_sum(taken + taken2, lane);
+            taken = lanes16_total(taken + taken2);
             float read = 0.f, read2 = 0.f;
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) {
-                float s = fmaf(write[r], value, decay[r] * S[r]);
-                s = fmaf(-removal[r], taken, s);
+                float s = fmaf(now.write[r], now.value, now.decay[r] * S[r]);
+                s = fmaf(-now.removal[r], taken, s);
                 S[r] = s;
-                if (r & 1) read2 = fmaf(s, read_by[r], read2);
-                else read = fmaf(s, read_by[r], read);
+                if (r & 1) read2 = fmaf(s, now.read_by[r], read2);
+                else read = fmaf(s, now.read_by[r], read);
             }
-            read = row16_sum(read + read2, lane);
+            read = lanes16_total(read + read2);
             if (lane == 0 && j < dv) out[((size_t)(t0 + tt) * heads + head) * dv + j] = read;
+        };
+        if (count == CHUNK) {
+#pragma unroll
+            for (int tt = 0; tt < CHUNK; ++tt) {
+                if (tt + 1 < CHUNK)
+                    rows[(tt + 1) & 1].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt + 1, lane, col, CHUNK * DKP, DKP);
+                one(tt, rows[tt & 1]);
+            }
+        } else {
+            for (int tt = 0; tt < count; ++tt) {
+                rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt, lane, col, CHUNK * DKP, DKP);
+                one(tt, rows[0]);
+            }
         }
         if (more) park(buffer ^ 1);
         __syncthreads();            // the other buffer is full; this one has been read
