@@ -75,18 +75,33 @@ __global__ __launch_bounds__(kWave) void general_delta_prepare_kernel(
 
 // Channel c of token t through the convolution: sum_j taps[c, K - 1 - j] x[t - j, c], where an input
 // from before the step comes from the request's tail (its last K - 1 inputs, oldest first).
+// KT: the number of taps where it is known when the kernel is built (all of a channel's loads are
+// then asked for together), 0: whatever K says.
+template <int KT>
 __device__ __forceinline__ float conv_at(const float* __restrict__ proj, size_t cols, int t, int local, int c,
                                          const float* __restrict__ taps, int K, const float* __restrict__ tail, int C) {
     float y = 0.f;
-    for (int j = 0; j < K; ++j) {
-        const float x = j <= local ? proj[(size_t)(t - j) * cols + c]
-                                   : tail[(size_t)((K - 1) - (j - local)) * C + c];
-        y = fmaf(taps[(size_t)c * K + (K - 1 - j)], x, y);
+    if constexpr (KT > 0) {
+        float x[KT], w[KT];
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            x[j] = j <= local ? proj[(size_t)(t - j) * cols + c] : tail[(size_t)((KT - 1) - (j - local)) * C + c];
+            w[j] = taps[(size_t)c * KT + (KT - 1 - j)];
+        }
+#pragma unroll
+        for (int j = 0; j < KT; ++j) y = fmaf(w[j], x[j], y);
+    } else {
+        for (int j = 0; j < K; ++j) {
+            const float x = j <= local ? proj[(size_t)(t - j) * cols + c]
+                                       : tail[(size_t)((K - 1) - (j - local)) * C + c];
+            y = fmaf(taps[(size_t)c * K + (K - 1 - j)], x, y);
+        }
     }
     return y;
 }
 
 // One wave per (token, head).  proj [T, C + nv + 2 heads]: q | k | v | gate | beta | rate.
+template <int KT>
 __global__ __launch_bounds__(kWave) void gated_delta_prepare_kernel(
     const float* __restrict__ proj, int T, int heads, int kv_heads, int dk, int dv, int K,
     const float* __restrict__ taps, const float* __restrict__ tails, const float* __restrict__ rate_log,
@@ -106,8 +121,8 @@ __global__ __launch_bounds__(kWave) void gated_delta_prepare_kernel(
         const int i = lane + kWave * e;
         q[e] = k[e] = 0.f;
         if (i < dk) {
-            q[e] = silu_f(conv_at(proj, cols, t, local, kv * dk + i, taps, K, tail, C));
-            k[e] = silu_f(conv_at(proj, cols, t, local, nk + kv * dk + i, taps, K, tail, C));
+            q[e] = silu_f(conv_at<KT>(proj, cols, t, local, kv * dk + i, taps, K, tail, C));
+            k[e] = silu_f(conv_at<KT>(proj, cols, t, local, nk + kv * dk + i, taps, K, tail, C));
         }
         qq = fmaf(q[e], q[e], qq);
         kk = fmaf(k[e], k[e], kk);
@@ -132,7 +147,7 @@ __global__ __launch_bounds__(kWave) void gated_delta_prepare_kernel(
     }
     for (int i = lane; i < dv; i += kWave)
         v_out[((size_t)t * heads + head) * dv + i] =
-            silu_f(conv_at(proj, cols, t, local, 2 * nk + head * dv + i, taps, K, tail, C));
+            silu_f(conv_at<KT>(proj, cols, t, local, 2 * nk + head * dv + i, taps, K, tail, C));
 }
 
 // A thread per (request, channel): the new tail is the last K - 1 of (old tail, the step's inputs).
@@ -203,7 +218,9 @@ struct TokenRows {
 // column (16 ROWS >= dk); the tokens' vectors pass through LDS in stages of CHUNK tokens, the next
 // stage on its way from memory into registers while this one is worked through.  The state lies in
 // memory as [slot, head, value, key]: a column's key rows in a row.
-template <int ROWS, int CHUNK>
+// DEEP: a token's vectors are read a token ahead (more registers, fewer waves a SIMD: for steps
+// of long portions; steps of lone tokens are bound by the states' trip to memory and want the waves).
+template <int ROWS, int CHUNK, bool DEEP>
 __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     const float* __restrict__ coef, const float* __restrict__ v, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, int T, int heads, int dk, int dv) {
@@ -262,8 +279,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
         if (more) fetch(t0 + CHUNK);
         // a token's vectors are read from LDS while the token before it is worked through: only the
         // state itself ties one token to the next
-        TokenRows<ROWS> rows[2];
-        rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], 0, lane, col, CHUNK * DKP, DKP);
+        TokenRows<ROWS> rows[DEEP ? 2 : 1];
+        if (DEEP) rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], 0, lane, col, CHUNK * DKP, DKP);
         auto one = [&](int tt, const TokenRows<ROWS>& now) {
             float taken = 0.f, taken2 = 0.f;
 #pragma unroll
@@ -284,12 +301,13 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
             read = lanes16_total(read + read2);
             if (lane == 0 && j < dv) out[((size_t)(t0 + tt) * heads + head) * dv + j] = read;
         };
-        if (count == CHUNK) {
+        if (DEEP && count == CHUNK) {
 #pragma unroll
             for (int tt = 0; tt < CHUNK; ++tt) {
                 if (tt + 1 < CHUNK)
-                    rows[(tt + 1) & 1].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt + 1, lane, col, CHUNK * DKP, DKP);
-                one(tt, rows[tt & 1]);
+                    rows[DEEP ? (tt + 1) & 1 : 0].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt + 1, lane, col,
+                                                       CHUNK * DKP, DKP);
+                one(tt, rows[DEEP ? tt & 1 : 0]);
             }
         } else {
             for (int tt = 0; tt < count; ++tt) {
@@ -344,9 +362,22 @@ LC_API int lc_gated_delta_prepare(const float* proj, int T, int heads, int kv_he
                  (tails || K == 1) && tail_slots >= 0,
              "gated_delta_prepare: null pointer");
     LC_CHECK((long long)T * heads < (1ll << 31), "gated_delta_prepare: too many heads");
-    gated_delta_prepare_kernel<<<T * heads, kWave, 0, stream>>>(proj, T, heads, kv_heads, dk, dv, K, taps, tails,
-                                                                rate_log, rate_bias, unit_eps, tok_req, q_offsets,
-                                                                slot_ids, coef, v_out);
+#define LC_PREPARE(KT)                                                                                              \
+    gated_delta_prepare_kernel<KT><<<T * heads, kWave, 0, stream>>>(proj, T, heads, kv_heads, dk, dv, K, taps, tails, \
+                                                                    rate_log, rate_bias, unit_eps, tok_req, q_offsets, \
+                                                                    slot_ids, coef, v_out)
+    switch (K) {
+        case 1: LC_PREPARE(1); break;
+        case 2: LC_PREPARE(2); break;
+        case 3: LC_PREPARE(3); break;
+        case 4: LC_PREPARE(4); break;
+        case 5: LC_PREPARE(5); break;
+        case 6: LC_PREPARE(6); break;
+        case 7: LC_PREPARE(7); break;
+        case 8: LC_PREPARE(8); break;
+        default: LC_PREPARE(0); break;
+    }
+#undef LC_PREPARE
     LC_LAUNCH_CHECK("gated_delta_prepare");
     return 0;
 }
@@ -371,9 +402,14 @@ LC_API int lc_delta_scan(const float* coef, const float* v, float* state, int sl
     LC_CHECK(coef && v && state && out && q_offsets && slot_ids, "delta_scan: null pointer");
     LC_CHECK(R <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for the grid");
     const dim3 grid((dv + SCAN_COLUMNS - 1) / SCAN_COLUMNS, heads, R);
+    const bool deep = T >= 16 * R;       // portions of prompts, mostly
 #define LC_SCAN(ROWS, CHUNK)                                                                                      \
-    delta_scan_kernel<ROWS, CHUNK><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets, slot_ids, T, \
-                                                                      heads, dk, dv)
+    if (deep)                                                                                                     \
+        delta_scan_kernel<ROWS, CHUNK, true><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets,   \
+                                                                                slot_ids, T, heads, dk, dv);      \
+    else                                                                                                          \
+        delta_scan_kernel<ROWS, CHUNK, false><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets,  \
+                                                                                 slot_ids, T, heads, dk, dv)
     if (dk <= 16) LC_SCAN(1, 16);
     else if (dk <= 32) LC_SCAN(2, 16);
     else if (dk <= 64) LC_SCAN(4, 16);
