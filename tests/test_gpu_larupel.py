@@ -87,7 +87,8 @@ def dev(*tensors):
 
 # ------------------------------------------------------------------ kernels alone
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,rows,branch", [(50, None, True), (192, None, False), (1030, [3, 0, 3], True), (7, [1], False)])
+@pytest.mark.parametrize("n,rows,branch", [(50, None, True), (192, None, False), (1030, [3, 0, 3], True), (7, [1], False),
+                                           (9000, None, True), (8200, [4, 1], False)])
 def test_layer_norm(dtype, n, rows, branch):
     g = torch.Generator().manual_seed(n)
     h = torch.randn(5, n, generator=g) * 3 + 1
