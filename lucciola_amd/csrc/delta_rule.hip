@@ -3,7 +3,7 @@
 //
 // The recurrence, per head, with the state S [key, value] and per token the vectors decay,
 // probe, removal, write, read over the key channels and the value v:
-//     S <- diag(decay) S - removal (probe^T S) + write v^T        (both terms read the old S)
+//     S <- diag(decay) S - removal (probe^T S) + write v^T        (probe^T S: of S as the last token left it)
 //     o  = S^T read
 // A column of S (one value channel) never meets another, so the work is shared out by columns:
 // a workgroup owns 16 columns of one head of one request and walks the request's tokens in
@@ -166,9 +166,7 @@ __global__ void conv_tail_update_kernel(const float* __restrict__ proj, int cols
     for (int m = 0; m < K - 1; ++m) tail[(size_t)m * C + c] = keep[m];
 }
 
-constexpr int SCAN_COLUMNS = 16;      // value channels of a workgroup
 constexpr int SCAN_LANES = 16;        // lanes that share a column's key rows: one DPP row
-constexpr int SCAN_THREADS = SCAN_COLUMNS * SCAN_LANES;
 
 // Sum over the 16 lanes of a DPP row, every lane getting a total: neighbours, then pairs, then the
 // quads by two rotations.  Lanes of different quads add the quads' sums in different orders, so
@@ -197,39 +195,73 @@ __device__ __forceinline__ void load_rows(float (&dst)[ROWS], const float* __res
     }
 }
 
+// Pointers into LDS, said to be so: through a plain pointer the compiler may fall back on flat
+// loads, which wait on the memory counter too, and a wait for one of them then waits for every
+// load of the next stage that is still on its way from memory.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* glb_ptr_t;
+typedef __attribute__((address_space(3))) float lds_f;
+typedef __attribute__((address_space(3))) const float lds_cf;
+typedef float float4_v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const float4_v lds_cf4;
+
+template <int ROWS>
+__device__ __forceinline__ void lds_rows(float (&dst)[ROWS], const float* generic) {
+    lds_cf* p = (lds_cf*)generic;
+    if constexpr (ROWS % 4 == 0) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+            const float4_v q = *(lds_cf4*)(p + r);
+            dst[r] = q.x; dst[r + 1] = q.y; dst[r + 2] = q.z; dst[r + 3] = q.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) dst[r] = p[r];
+    }
+}
+
 // What a lane needs of one token: its run of each of the five vectors, and its column's value.
 template <int ROWS>
 struct TokenRows {
     float decay[ROWS], probe[ROWS], removal[ROWS], write[ROWS], read_by[ROWS], value;
     // stage: the stage's vectors [5][CHUNK][DKP] (`plane` floats a vector, `dkp` a token), values: [CHUNK][columns]
     __device__ __forceinline__ void load(const float* stage, const float* values, int tt, int lane, int col, int plane,
-                                         int dkp) {
+                                         int dkp, int columns) {
         const float* at = stage + tt * dkp + lane * ROWS;
-        load_rows<ROWS>(probe, at + plane);
-        load_rows<ROWS>(decay, at);
-        load_rows<ROWS>(removal, at + 2 * plane);
-        load_rows<ROWS>(write, at + 3 * plane);
-        load_rows<ROWS>(read_by, at + 4 * plane);
-        value = values[tt * SCAN_COLUMNS + col];
+        lds_rows<ROWS>(probe, at + plane);
+        lds_rows<ROWS>(decay, at);
+        lds_rows<ROWS>(removal, at + 2 * plane);
+        lds_rows<ROWS>(write, at + 3 * plane);
+        lds_rows<ROWS>(read_by, at + 4 * plane);
+        value = ((lds_cf*)values)[tt * columns + col];
     }
 };
 
-// grid (column blocks, heads, requests).  A lane holds the ROWS key rows lane * ROWS ... of its
-// column (16 ROWS >= dk); the tokens' vectors pass through LDS in stages of CHUNK tokens, the next
-// stage on its way from memory into registers while this one is worked through.  The state lies in
-// memory as [slot, head, value, key]: a column's key rows in a row.
+// grid (column blocks, heads, requests); a workgroup owns COLS value channels (16 lanes each).  A
+// lane holds the ROWS key rows lane * ROWS ... of its column (16 ROWS >= dk); the tokens' vectors pass
+// through LDS in stages of CHUNK tokens.  Where the key rows fill a stage's rows (dk = 16 ROWS) the
+// stages are a ring that loads from memory fill directly, two stages ahead of the one being worked
+// through (a stage's trip takes about 2 us, its eight tokens' work a little more); else the next stage
+// travels through registers.  The state lies in memory as [slot, head, value, key]: a column's key
+// rows in a row.  (Workgroups of four columns, one wave each, were measured too: 1,020 us against
+// 594 for a 2,048-token request of 16 heads of 128 x 128.)
 // DEEP: a token's vectors are read a token ahead (more registers, fewer waves a SIMD: for steps
 // of long portions; steps of lone tokens are bound by the states' trip to memory and want the waves).
-template <int ROWS, int CHUNK, bool DEEP>
-__global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
+template <int ROWS, int CHUNK, bool DEEP, int COLS>
+__global__ __launch_bounds__(COLS * SCAN_LANES) void delta_scan_kernel(
     const float* __restrict__ coef, const float* __restrict__ v, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, int T, int heads, int dk, int dv) {
+    constexpr int SCAN_COLUMNS = COLS, SCAN_THREADS = COLS * SCAN_LANES;
     constexpr int DKP = ROWS * SCAN_LANES;                 // key rows with padding
     constexpr int VEC = 5 * CHUNK * DKP;                   // floats of a stage's vectors
     constexpr int PER_THREAD = VEC / SCAN_THREADS;
     static_assert(VEC % SCAN_THREADS == 0 && CHUNK * SCAN_COLUMNS <= SCAN_THREADS, "stage does not fit the threads");
-    __shared__ __attribute__((aligned(16))) float vec[2][5][CHUNK][DKP];
-    __shared__ float val[2][CHUNK][SCAN_COLUMNS];
+    // stages in LDS: a ring of three; the loads that go through registers use two of them
+    constexpr int NS = 3, AHEAD = NS - 1;
+    __shared__ __attribute__((aligned(16))) float vec[NS][5][CHUNK][DKP];
+    // a stage's values [CHUNK][COLS], in a slot of whole 64-lane loads
+    constexpr int VAL_SLOT = ((CHUNK * COLS + kWave - 1) / kWave) * kWave;
+    __shared__ __attribute__((aligned(16))) float val[NS][VAL_SLOT];
     const int tid = threadIdx.x;
     const int col = tid / SCAN_LANES, lane = tid % SCAN_LANES;
     const int head = blockIdx.y, req = blockIdx.z;
@@ -262,25 +294,46 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
             next_val = (tt < count && jj < dv) ? v[((size_t)(t0 + tt) * heads + head) * dv + jj] : 0.f;
         }
     };
-    auto park = [&](int buffer) {
-        float* flat = &vec[buffer][0][0][0];
+    auto park = [&](int buffer, bool vectors) {
+        lds_f* flat = (lds_f*)&vec[buffer][0][0][0];
+        if (vectors) {
 #pragma unroll
-        for (int k = 0; k < PER_THREAD; ++k) flat[tid + k * SCAN_THREADS] = next_vec[k];
-        if (tid < CHUNK * SCAN_COLUMNS) val[buffer][tid / SCAN_COLUMNS][tid % SCAN_COLUMNS] = next_val;
+            for (int k = 0; k < PER_THREAD; ++k) flat[tid + k * SCAN_THREADS] = next_vec[k];
+        }
+        if (tid < CHUNK * SCAN_COLUMNS) ((lds_f*)&val[buffer][0])[tid] = next_val;
+    };
+    // Where the key rows fill a stage's rows without padding (dk = 16 ROWS), the vectors go from memory
+    // straight into LDS, 16 bytes a lane and 1 KB an instruction, past the registers: nothing of the
+    // token loop waits for them.  A token behind the request's end is its last token once more.
+    constexpr int DIRECT_LOADS = VEC / 256;
+    constexpr bool CAN_DIRECT = VEC % 256 == 0;
+    const bool direct = CAN_DIRECT && dk == DKP;
+    auto fetch_direct = [&](int t0, int buffer) {
+        const int wave = tid / kWave, lane64 = tid % kWave;
+        for (int idx = wave; idx < DIRECT_LOADS; idx += SCAN_THREADS / kWave) {
+            const int f = idx * 256 + lane64 * 4;
+            const int i = f % DKP, tt = (f / DKP) % CHUNK, c = f / (DKP * CHUNK);
+            const int t = min(t0 + tt, last - 1);
+            const float* src = coef + c * plane + ((size_t)t * heads + head) * dk + i;
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)src, (lds_ptr_t)(&vec[buffer][0][0][0] + idx * 256), 16, 0, 0);
+        }
+        // the values, four bytes a lane (a column behind dv reads the last one's: it is never written)
+        for (int idx = wave; idx * kWave < CHUNK * SCAN_COLUMNS; idx += SCAN_THREADS / kWave) {
+            const int f = idx * kWave + lane64;
+            const int cc = f % SCAN_COLUMNS, tt = min(f / SCAN_COLUMNS, CHUNK - 1);
+            const int jj = min(blockIdx.x * SCAN_COLUMNS + cc, dv - 1);
+            const int t = min(t0 + tt, last - 1);
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(v + ((size_t)t * heads + head) * dv + jj),
+                                             (lds_ptr_t)(&val[buffer][0] + idx * kWave), 4, 0, 0);
+        }
     };
 
-    fetch(first);
-    park(0);
-    __syncthreads();
-    int buffer = 0;
-    for (int t0 = first; t0 < last; t0 += CHUNK, buffer ^= 1) {
-        const int count = min(CHUNK, last - t0);
-        const bool more = t0 + CHUNK < last;
-        if (more) fetch(t0 + CHUNK);
+    // a stage's tokens, one after the other, from LDS stage `buffer`
+    auto work = [&](int buffer, int t0, int count) {
         // a token's vectors are read from LDS while the token before it is worked through: only the
         // state itself ties one token to the next
         TokenRows<ROWS> rows[DEEP ? 2 : 1];
-        if (DEEP) rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], 0, lane, col, CHUNK * DKP, DKP);
+        if (DEEP) rows[0].load(&vec[buffer][0][0][0], &val[buffer][0], 0, lane, col, CHUNK * DKP, DKP, COLS);
         auto one = [&](int tt, const TokenRows<ROWS>& now) {
             float taken = 0.f, taken2 = 0.f;
 #pragma unroll
@@ -305,18 +358,49 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
 #pragma unroll
             for (int tt = 0; tt < CHUNK; ++tt) {
                 if (tt + 1 < CHUNK)
-                    rows[DEEP ? (tt + 1) & 1 : 0].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt + 1, lane, col,
-                                                       CHUNK * DKP, DKP);
+                    rows[DEEP ? (tt + 1) & 1 : 0].load(&vec[buffer][0][0][0], &val[buffer][0], tt + 1, lane, col,
+                                                       CHUNK * DKP, DKP, COLS);
                 one(tt, rows[DEEP ? tt & 1 : 0]);
             }
         } else {
             for (int tt = 0; tt < count; ++tt) {
-                rows[0].load(&vec[buffer][0][0][0], &val[buffer][0][0], tt, lane, col, CHUNK * DKP, DKP);
+                rows[0].load(&vec[buffer][0][0][0], &val[buffer][0], tt, lane, col, CHUNK * DKP, DKP, COLS);
                 one(tt, rows[0]);
             }
         }
-        if (more) park(buffer ^ 1);
-        __syncthreads();            // the other buffer is full; this one has been read
+    };
+    if (direct) {
+        // the ring: AHEAD stages are on their way while one is worked through.  The memory counter
+        // counts a wave's loads (and its stores of read-outs, which only makes the wait stricter) in
+        // order: when at most the loads of the AHEAD - 1 youngest stages are left, the next stage is there.
+        constexpr int PER_WAVE = DIRECT_LOADS / (SCAN_THREADS / kWave);
+        constexpr int LEFT = (AHEAD - 1) * PER_WAVE < 63 ? (AHEAD - 1) * PER_WAVE : 63;
+        for (int a = 0; a < AHEAD; ++a)
+            if (first + a * CHUNK < last) fetch_direct(first + a * CHUNK, a);
+        if (first + (AHEAD - 1) * CHUNK < last) wait_vmcnt<LEFT>();     // all AHEAD stages were asked for
+        else wait_vmcnt<0>();
+        __syncthreads();
+        int buffer = 0;
+        for (int t0 = first; t0 < last; t0 += CHUNK, buffer = buffer + 1 == NS ? 0 : buffer + 1) {
+            if (t0 + AHEAD * CHUNK < last) fetch_direct(t0 + AHEAD * CHUNK, (buffer + AHEAD) % NS);
+            work(buffer, t0, min(CHUNK, last - t0));
+            // the youngest stages may still travel; none is asked for beyond the request's end
+            if (t0 + AHEAD * CHUNK < last) wait_vmcnt<LEFT>();
+            else wait_vmcnt<0>();
+            __syncthreads();        // the next stage is there; this one has been read
+        }
+    } else {
+        fetch(first);
+        park(0, true);
+        __syncthreads();
+        int buffer = 0;
+        for (int t0 = first; t0 < last; t0 += CHUNK, buffer ^= 1) {
+            const bool more = t0 + CHUNK < last;
+            if (more) fetch(t0 + CHUNK);
+            work(buffer, t0, min(CHUNK, last - t0));
+            if (more) park(buffer ^ 1, true);
+            __syncthreads();        // the other stage is full; this one has been read
+        }
     }
     if (whole) {
 #pragma unroll
@@ -401,20 +485,20 @@ LC_API int lc_delta_scan(const float* coef, const float* v, float* state, int sl
     if (R == 0 || T == 0) return 0;
     LC_CHECK(coef && v && state && out && q_offsets && slot_ids, "delta_scan: null pointer");
     LC_CHECK(R <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for the grid");
-    const dim3 grid((dv + SCAN_COLUMNS - 1) / SCAN_COLUMNS, heads, R);
     const bool deep = T >= 16 * R;       // portions of prompts, mostly
-#define LC_SCAN(ROWS, CHUNK)                                                                                      \
-    if (deep)                                                                                                     \
-        delta_scan_kernel<ROWS, CHUNK, true><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets,   \
-                                                                                slot_ids, T, heads, dk, dv);      \
-    else                                                                                                          \
-        delta_scan_kernel<ROWS, CHUNK, false><<<grid, SCAN_THREADS, 0, stream>>>(coef, v, state, out, q_offsets,  \
-                                                                                 slot_ids, T, heads, dk, dv)
+    const dim3 grid((dv + 15) / 16, heads, R);
+#define LC_SCAN_AS(ROWS, CHUNK, DEEP, COLS)                                                                          \
+    delta_scan_kernel<ROWS, CHUNK, DEEP, COLS><<<grid, COLS * SCAN_LANES, 0, stream>>>(coef, v, state, out, q_offsets, \
+                                                                                       slot_ids, T, heads, dk, dv)
+#define LC_SCAN(ROWS, CHUNK)                          \
+    if (deep) LC_SCAN_AS(ROWS, CHUNK, true, 16);      \
+    else LC_SCAN_AS(ROWS, CHUNK, false, 16)
     if (dk <= 16) LC_SCAN(1, 16);
     else if (dk <= 32) LC_SCAN(2, 16);
     else if (dk <= 64) LC_SCAN(4, 16);
     else if (dk <= 128) LC_SCAN(8, 8);
     else LC_SCAN(16, 4);
+#undef LC_SCAN_AS
 #undef LC_SCAN
     LC_LAUNCH_CHECK("delta_scan");
     return 0;

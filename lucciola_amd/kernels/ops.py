@@ -1506,7 +1506,7 @@ def conv_tail_update(proj: torch.Tensor, tail: torch.Tensor, channels: int, num_
 def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offsets: torch.Tensor,
                slot_ids: torch.Tensor, num_requests: int, heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The delta-rule recurrence over every request's tokens in order, per head:
-    ``S <- diag(decay) S - removal (probe^T S) + write v^T`` (both terms read the old S), ``o = S^T read``.
+    ``S <- diag(decay) S - removal (probe^T S) + write v^T`` (the probe meets S as the last token left it, before the decay), ``o = S^T read``.
     ``coef`` float32 [5, T, heads key_dim] holds decay, probe, removal, write, read; ``v`` float32
     [T, heads value_dim]; ``state`` float32 [slots, heads, value_dim, key_dim] (S transposed: a value
     channel's key rows lie in a row) is read at the request's slot before its first token of the step

@@ -6,7 +6,7 @@ Both are instances of one recurrence per head (``ops.delta_scan``; in memory the
 transposed, [slot, head, value, key], and only that kernel reads it), with the state S [key, value]
 and, per token, five vectors over the key channels and the value v:
 
-    S <- diag(decay) S - removal (probe^T S) + write v^T        (both terms read the old S)
+    S <- diag(decay) S - removal (probe^T S) + write v^T        (probe^T S: of S as the last token left it)
     o  = S^T read
 
 ``general_delta`` (the generalized delta rule): decay w = exp(-c sigmoid(W2 tanh(W1 h) + w0)) per

@@ -152,7 +152,7 @@ def gated_delta_mixer(h, weights, p, m, eps):
 
 def general_delta_mixer(h, weights, p, m, eps):
     """Per head, token by token, with the unit key u = k / sqrt(sum k^2 + 1e-6):
-    S <- diag(w) S - (a u)(u^T S) + k v^T (both terms read the old S); o = S^T r."""
+    S <- diag(w) S - (a u)(u^T S) + k v^T (u^T S is taken of S before its decay); o = S^T r."""
     T = h.shape[0]
     H, d = m["heads"], m["dim"]
     r = linear(h, weights[p + "r"]).view(T, H, d)
