@@ -362,16 +362,19 @@ def design_configs(name, routed):
     return qwen, pubodra
 
 
-def larupel_design_config(name):
+def larupel_design_config(name, routed=True):
     """The Larupel decoder at the same width, heads, head size, feed-forward width, vocabulary and
     depth: attention, the generalized delta rule, the gated delta rule and a second attention layer
     that reads the first one's keys and values; the two recurrent layers have routed feed-forwards
-    (4 of 32 experts of ff / 4 and a shared one of ff / 4), the attention layers dense ones."""
+    (4 of 32 experts of ff / 4 and a shared one of ff / 4; ``routed`` False: dense ones), the
+    attention layers dense ones."""
     width, heads, ff = DESIGN_SIZES[name]
     kv = max(1, heads // 4)
     attention = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
     dense = {"kind": "dense", "ff": ff}
     moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
+    if not routed:
+        moe = dense
     layers = [{"type": "attention", "mixer": attention, "mlp": dense},
               {"type": "general_delta", "mixer": {"heads": heads, "dim": 128}, "mlp": moe},
               {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "conv": 4}, "mlp": moe},
@@ -462,11 +465,12 @@ def designs_workload(args, dev):
                 results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
                                           args.design_context, args.steps)
                 say(f"{key}: {results[key]}")
-        if "larupel" in wanted:
-            key = f"{name}/larupel"
-            results[key] = design_run(larupel_design_config(name), dtype, dev, args.block_size, args.prefill_tokens,
-                                      batches, args.design_context, args.steps)
-            say(f"{key}: {results[key]}")
+        for model in ("larupel", "larupel_dense"):
+            if model in wanted:
+                key = f"{name}/{model}"
+                results[key] = design_run(larupel_design_config(name, routed=model == "larupel"), dtype, dev,
+                                          args.block_size, args.prefill_tokens, batches, args.design_context, args.steps)
+                say(f"{key}: {results[key]}")
     head = f"decode_b{batches[0]}_ctx{args.design_context}"
     key = ([k for k in results if "pubodra_dense" in k] or list(results))[0]
     line = {"metric": f"decode tok/s ({key.split('/')[1]}, {key.split('/')[0]}, {DESIGN_LAYERS} layers, batch {batches[0]}, "
@@ -514,7 +518,7 @@ def main() -> int:
     ap.add_argument("--design-sizes", default="w2048,w4096", help="designs: which of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-batches", default="8,64", help="designs: decode batch sizes")
     ap.add_argument("--design-models", default="qwen3,pubodra_dense,pubodra_routed,larupel",
-                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel")
+                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel, larupel_dense")
     ap.add_argument("--design-context", type=int, default=2048, help="designs: tokens a decoding request holds")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "designs"],
                     help="decode: the default line; mixed: only the 0.6B-shaped mixed workload, as a line of its own")

@@ -256,8 +256,9 @@ __global__ __launch_bounds__(COLS * SCAN_LANES) void delta_scan_kernel(
     constexpr int VEC = 5 * CHUNK * DKP;                   // floats of a stage's vectors
     constexpr int PER_THREAD = VEC / SCAN_THREADS;
     static_assert(VEC % SCAN_THREADS == 0 && CHUNK * SCAN_COLUMNS <= SCAN_THREADS, "stage does not fit the threads");
-    // stages in LDS: a ring of three; the loads that go through registers use two of them
-    constexpr int NS = 3, AHEAD = NS - 1;
+    // stages in LDS: a ring of three for long portions, two for steps of lone tokens (less LDS, more
+    // workgroups a CU); the loads that go through registers use two of them
+    constexpr int NS = DEEP ? 3 : 2, AHEAD = NS - 1;
     __shared__ __attribute__((aligned(16))) float vec[NS][5][CHUNK][DKP];
     // a stage's values [CHUNK][COLS], in a slot of whole 64-lane loads
     constexpr int VAL_SLOT = ((CHUNK * COLS + kWave - 1) / kWave) * kWave;
