@@ -197,7 +197,9 @@ def test_gated_delta_prepare_and_tail(heads, kv, dk, dv, K):
 
 
 @pytest.mark.parametrize("heads,dk,dv,lengths", [(2, 16, 16, [5, 1, 40]), (3, 7, 9, [1, 1, 1, 1]), (2, 32, 64, [70]),
-                                                 (1, 64, 20, [3, 33]), (2, 130, 17, [18, 2]), (1, 128, 128, [9])])
+                                                 (1, 64, 20, [3, 33]), (2, 130, 17, [18, 2]), (1, 128, 128, [9]),
+                                                 (2, 128, 48, [100, 3]), (1, 256, 16, [40]), (1, 200, 16, [37]),
+                                                 (3, 16, 5, [1, 50, 2])])
 def test_delta_scan(heads, dk, dv, lengths):
     g = torch.Generator().manual_seed(dk + dv)
     T, R = sum(lengths), len(lengths)
