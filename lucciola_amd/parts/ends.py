@@ -8,7 +8,8 @@ parts like any other, so that an architecture with a scaled embedding, a head wi
 capped logits registers its own kind and the model class stays as it is.
 
 Interfaces:
-  Embedding   declare() -> {"weight": ...}; forward(ids int32 [T]) -> float32 [T, H];
+  Embedding   declare() -> {"weight": ...}; forward(ids int32 [T]) -> float32 [T, H]
+              (forward(ids, positions int32 [T]) where the part sets takes_positions);
               table() -> the tensor a tied head shares
   Head        declare() (nothing when tied); bind(tensors, ctx, shared=table or None);
               forward(x act [R, H]) -> float32 [R, V]

@@ -212,3 +212,22 @@ def test_greedy_generation_through_the_scheduler(monkeypatch):
     assert got == [plain_larupel.greedy(cfg, weights, p, 5) for p in prompts]
     engine.runner.cache.check()
     assert not engine.runner.cache.requests
+
+
+def test_the_bench_configurations_are_models_of_the_design():
+    """What ``bench.py --workload designs`` builds for this design reads as a configuration, with the
+    sizes of the model beside it."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(os.path.dirname(
+        os.path.abspath(__file__))), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for name, (width, heads, ff) in bench.DESIGN_SIZES.items():
+        for routed in (True, False):
+            cfg = LarupelConfig.from_dict(bench.larupel_design_config(name, routed=routed))
+            assert (cfg.width, cfg.vocab, len(cfg.layers)) == (width, bench.DESIGN_VOCAB, bench.DESIGN_LAYERS)
+            assert [l.type for l in cfg.layers] == ["attention", "general_delta", "delta", "attention"]
+            assert cfg.layers[3].mixer.kv_from == 0 and cfg.layers[0].mixer.heads == heads
+            assert [l.mlp.kind for l in cfg.layers] == (["dense", "moe", "moe", "dense"] if routed else ["dense"] * 4)
+            declared_tensors(larupel_model_spec(cfg))
