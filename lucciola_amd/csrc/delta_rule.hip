@@ -180,7 +180,7 @@ __device__ __forceinline__ float lanes16_total(float v) {
     return v;
 }
 
-// ROWS floats from LDS or memory that is 16-byte aligned where ROWS is a multiple of four.
+// ROWS floats from memory that is 16-byte aligned where ROWS is a multiple of four (the state's rows).
 template <int ROWS>
 __device__ __forceinline__ void load_rows(float (&dst)[ROWS], const float* __restrict__ p) {
     if constexpr (ROWS % 4 == 0) {
