@@ -524,6 +524,41 @@ def test_float32_logits_do_not_depend_on_the_cut():
             assert torch.equal(row, other[key]), f"{key}: the bits differ between two cuts"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_a_batch_of_unequal_requests_against_each_alone(key, dtype):
+    """Four requests of unequal length in one step, then a step of lone tokens beside a portion: every
+    row against the same request run alone (the same bits in float32; within rounding in bfloat16,
+    where other rows in a step mean other product kernels)."""
+    cfg, page, weights, prompts, refs = case(key)
+    names = list(prompts)[:4]
+    alone = {}
+    for n in names:
+        runner = make_runner(cfg, weights, page, 64, dtype, DEV)
+        alone.update(replay(runner, traces.whole({n: prompts[n]})))
+    runner = make_runner(cfg, weights, page, 64, dtype, DEV)
+    cut = {n: max(1, len(prompts[n]) - 3) for n in names}
+    steps = [([(n, prompts[n][:cut[n]], list(range(cut[n]))) for n in names], [])]
+    rest = {n: prompts[n][cut[n]:] for n in names}
+    longest = max(len(r) for r in rest.values())
+    for k in range(longest):
+        entries = [(n, [rest[n][k]], [0]) for n in names if k < len(rest[n])]
+        steps.append((entries, [n for n in names if k == len(rest[n]) - 1]))
+    together = replay(runner, [s for s in steps if s[0]])
+    assert sorted(together) == sorted(alone)
+    errors = []
+    for row_key, row in alone.items():
+        if dtype == "float32":
+            assert torch.equal(row, together[row_key]), f"{row_key}: the bits differ between alone and in a batch"
+        else:
+            diff = row - together[row_key]
+            errors.append(float((diff - diff.mean()).pow(2).mean().sqrt() / (row - row.mean()).pow(2).mean().sqrt()))
+    if errors:      # a router's close call may fall the other way in a few rows
+        errors.sort()
+        assert errors[len(errors) // 2] < 0.03, f"median difference {errors[len(errors) // 2]:.3e}"
+        assert sum(e > 0.1 for e in errors) <= len(errors) // 10
+
+
 def _random_config(rng):
     width = rng.choice([24, 40, 64, 72])
     layers, lenders = [], []
